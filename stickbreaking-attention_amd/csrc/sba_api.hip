@@ -1,0 +1,219 @@
+// C ABI of libsba: argument validation, workspace layout and kernel launches.  See include/sba.h.
+#include <hip/hip_runtime.h>
+
+#include "../../include/sba.h"
+#include "sba_params.hpp"
+
+namespace sba {
+hipError_t launch_sched(const SchedParams& p, hipStream_t stream);
+hipError_t launch_fwd(const FwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
+hipError_t launch_bwd_dq(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
+hipError_t launch_bwd_dkv(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
+hipError_t launch_fwd_f32(const FwdParams& p, int max_tiles, hipStream_t stream);
+hipError_t launch_bwd_f32(const BwdParams& p, int max_q_tiles, int max_k_tiles, hipStream_t stream);
+}  // namespace sba
+
+namespace {
+
+constexpr double kLog2e = 1.4426950408889634;
+constexpr int kBlockQ = 128, kBlockK = 64;
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+struct Layout {
+  int64_t max_q_tiles, max_k_tiles, carry_slots_per_head;
+  size_t off_counts, off_q_tiles, off_k_tiles, off_carry_base, off_prefix;
+  size_t fwd_bytes, bwd_bytes, carry_bytes;
+};
+
+int plan(const SbaArgs* a, Layout* out) {
+  if (a->num_heads <= 0 || a->num_seqs <= 0 || a->total_tokens <= 0) return SBA_ERR_SHAPE;
+  if (a->head_dim < 1 || a->head_dim > 128) return SBA_ERR_HEAD_DIM;
+  if (a->dtype != SBA_BF16 && a->dtype != SBA_F16 && a->dtype != SBA_F32) return SBA_ERR_DTYPE;
+  if (a->total_tokens > (int64_t)1 << 30) return SBA_ERR_SHAPE;
+  Layout L{};
+  const int64_t T = a->total_tokens, B = a->num_seqs;
+  const bool fixed = a->cu_seqlens == nullptr;
+  int64_t max_len = (a->max_seqlen > 0 && a->max_seqlen < T) ? a->max_seqlen : T;
+  if (fixed) {
+    L.max_q_tiles = B * cdiv(T, kBlockQ);
+    L.max_k_tiles = B * cdiv(T, kBlockK);
+    L.carry_slots_per_head = B * sba::carry_slots(cdiv(T, kBlockQ));
+  } else {
+    L.max_q_tiles = cdiv(T, kBlockQ) + B;
+    L.max_k_tiles = cdiv(T, kBlockK) + B;
+    // sum_s 128 M_s (M_s + 1) with M_s <= L_s/128 + 1 and sum_s L_s^2 <= T * max_len
+    L.carry_slots_per_head = cdiv(T * max_len, 128) + 3 * T + 256 * B;
+  }
+  size_t off = 0;
+  L.off_counts = off;      off = align_up(off + 256, 256);
+  L.off_q_tiles = off;     off = align_up(off + (size_t)L.max_q_tiles * sizeof(sba::Tile), 256);
+  L.off_carry_base = off;  off = align_up(off + (size_t)B * sizeof(int64_t), 256);
+  L.fwd_bytes = off;
+  L.off_k_tiles = off;     off = align_up(off + (size_t)L.max_k_tiles * sizeof(sba::Tile), 256);
+  L.carry_bytes = align_up((size_t)L.carry_slots_per_head * a->num_heads * sizeof(float), 256);
+  L.off_prefix = off;      off += L.carry_bytes;
+  L.bwd_bytes = off;
+  *out = L;
+  return SBA_OK;
+}
+
+size_t elem_size(int dtype) { return dtype == SBA_F32 ? 4 : 2; }
+
+// A tensor is usable with 16-byte accesses when its base and its row/head/batch strides are 16-byte multiples.
+bool vec16(const SbaTensor& t, size_t es, bool fixed) {
+  const int64_t per = 16 / (int64_t)es;
+  if (((uintptr_t)t.ptr & 15) != 0) return false;
+  if (t.stride_token % per || t.stride_head % per) return false;
+  if (fixed && (t.stride_batch % per)) return false;
+  return true;
+}
+int check_tensor(const SbaTensor& t, bool required, bool fixed) {
+  if (!t.ptr) return required ? SBA_ERR_NULL : SBA_OK;
+  if (t.stride_token < 0 || t.stride_head < 0 || (fixed && t.stride_batch < 0)) return SBA_ERR_STRIDE;
+  return SBA_OK;
+}
+sba::TensorRef ref(const SbaTensor& t, bool fixed) { return sba::TensorRef{t.ptr, fixed ? t.stride_batch : 0, t.stride_head, t.stride_token}; }
+sba::VectorRef vref(const SbaVector& t, bool fixed) { return sba::VectorRef{t.ptr, fixed ? t.stride_batch : 0, t.stride_head, t.stride_token}; }
+
+int run_sched(const SbaArgs* a, const Layout& L, bool want_key_tiles, bool want_carry_base, hipStream_t stream) {
+  char* ws = (char*)a->workspace;
+  sba::SchedParams sp{};
+  sp.cu = a->cu_seqlens;
+  sp.cu_is_int64 = a->cu_is_int64;
+  sp.cu_has_leading_zero = a->cu_has_leading_zero;
+  sp.num_seqs = a->num_seqs;
+  sp.fixed_len = (int32_t)a->total_tokens;
+  sp.attend_current = a->attend_current ? 1 : 0;
+  sp.want_key_tiles = want_key_tiles ? 1 : 0;
+  sp.want_carry_base = want_carry_base ? 1 : 0;
+  sp.q_tiles = (sba::Tile*)(ws + L.off_q_tiles);
+  sp.k_tiles = (sba::Tile*)(ws + L.off_k_tiles);
+  sp.counts = (int32_t*)(ws + L.off_counts);
+  sp.carry_base = (int64_t*)(ws + L.off_carry_base);
+  return sba::launch_sched(sp, stream) == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sba_version(void) { return SBA_VERSION; }
+
+const char* sba_strerror(int status) {
+  switch (status) {
+    case SBA_OK: return "ok";
+    case SBA_ERR_NULL: return "a required pointer is NULL";
+    case SBA_ERR_DTYPE: return "unsupported dtype";
+    case SBA_ERR_HEAD_DIM: return "head_dim must be in 1..128";
+    case SBA_ERR_STRIDE: return "negative or unsupported stride";
+    case SBA_ERR_ALIGN: return "tensor base pointer is not aligned to its element size";
+    case SBA_ERR_SHAPE: return "sizes must be positive (and total_tokens <= 2^30)";
+    case SBA_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+    case SBA_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown status";
+  }
+}
+
+int sba_workspace_bytes(const SbaArgs* args, size_t* fwd_bytes, size_t* bwd_bytes, size_t* carry_bytes) {
+  if (!args) return SBA_ERR_NULL;
+  Layout L;
+  const int st = plan(args, &L);
+  if (st != SBA_OK) return st;
+  if (fwd_bytes) *fwd_bytes = L.fwd_bytes;
+  if (bwd_bytes) *bwd_bytes = L.bwd_bytes;
+  if (carry_bytes) *carry_bytes = L.carry_bytes;
+  return SBA_OK;
+}
+
+int sba_fwd(const SbaArgs* a) {
+  if (!a) return SBA_ERR_NULL;
+  Layout L;
+  int st = plan(a, &L);
+  if (st != SBA_OK) return st;
+  const bool fixed = a->cu_seqlens == nullptr;
+  const size_t es = elem_size(a->dtype);
+  if ((st = check_tensor(a->q, true, fixed)) || (st = check_tensor(a->k, true, fixed)) ||
+      (st = check_tensor(a->v, true, fixed)) || (st = check_tensor(a->o, true, fixed)))
+    return st;
+  if (!a->rem.ptr || !a->row_stat) return SBA_ERR_NULL;
+  for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->o})
+    if (t->ptr && ((uintptr_t)t->ptr % es)) return SBA_ERR_ALIGN;
+  if (!a->workspace || ((uintptr_t)a->workspace & 255) || a->workspace_bytes < L.fwd_bytes) return SBA_ERR_WORKSPACE;
+  hipStream_t stream = (hipStream_t)a->stream;
+  if ((st = run_sched(a, L, false, a->carry != nullptr, stream)) != SBA_OK) return st;
+
+  char* ws = (char*)a->workspace;
+  sba::FwdParams p{};
+  p.q = ref(a->q, fixed); p.k = ref(a->k, fixed); p.v = ref(a->v, fixed); p.o = ref(a->o, fixed);
+  p.rem = vref(a->rem, fixed);
+  p.row_stat = a->row_stat;
+  p.carry = a->carry;
+  p.carry_base = (const int64_t*)(ws + L.off_carry_base);
+  p.carry_head_stride = L.carry_slots_per_head;
+  p.stat_sb = fixed ? (int64_t)a->num_heads * a->total_tokens : 0;
+  p.stat_sh = a->total_tokens;
+  p.tiles = (const sba::Tile*)(ws + L.off_q_tiles);
+  p.counts = (const int32_t*)(ws + L.off_counts);
+  p.num_heads = a->num_heads;
+  p.head_dim = a->head_dim;
+  p.scale_log2 = (float)((double)a->logit_scale * kLog2e);
+  p.attend_current = a->attend_current ? 1 : 0;
+  bool v16 = (a->head_dim % (16 / (int)es)) == 0;
+  for (const SbaTensor* t : {&a->q, &a->k, &a->v}) v16 = v16 && vec16(*t, es, fixed);
+  p.vec_ok = v16 ? 1 : 0;
+  hipError_t e = (a->dtype == SBA_F32) ? sba::launch_fwd_f32(p, (int)L.max_q_tiles, stream)
+                                       : sba::launch_fwd(p, a->dtype == SBA_F16, (int)L.max_q_tiles, stream);
+  return e == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
+}
+
+int sba_bwd(const SbaArgs* a) {
+  if (!a) return SBA_ERR_NULL;
+  Layout L;
+  int st = plan(a, &L);
+  if (st != SBA_OK) return st;
+  const bool fixed = a->cu_seqlens == nullptr;
+  const size_t es = elem_size(a->dtype);
+  if ((st = check_tensor(a->q, true, fixed)) || (st = check_tensor(a->k, true, fixed)) ||
+      (st = check_tensor(a->v, true, fixed)) || (st = check_tensor(a->d_o, true, fixed)) ||
+      (st = check_tensor(a->dq, true, fixed)) || (st = check_tensor(a->dk, true, fixed)) ||
+      (st = check_tensor(a->dv, true, fixed)))
+    return st;
+  if (!a->carry) return SBA_ERR_NULL;
+  for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
+    if (t->ptr && ((uintptr_t)t->ptr % es)) return SBA_ERR_ALIGN;
+  if (!a->workspace || ((uintptr_t)a->workspace & 255) || a->workspace_bytes < L.bwd_bytes) return SBA_ERR_WORKSPACE;
+  hipStream_t stream = (hipStream_t)a->stream;
+  if ((st = run_sched(a, L, true, true, stream)) != SBA_OK) return st;
+
+  char* ws = (char*)a->workspace;
+  sba::BwdParams p{};
+  p.q = ref(a->q, fixed); p.k = ref(a->k, fixed); p.v = ref(a->v, fixed);
+  p.d_o = ref(a->d_o, fixed);
+  p.dq = ref(a->dq, fixed); p.dk = ref(a->dk, fixed); p.dv = ref(a->dv, fixed);
+  p.d_rem = vref(a->d_rem, fixed);
+  p.q_tiles = (const sba::Tile*)(ws + L.off_q_tiles);
+  p.k_tiles = (const sba::Tile*)(ws + L.off_k_tiles);
+  p.counts = (const int32_t*)(ws + L.off_counts);
+  p.carry_base = (const int64_t*)(ws + L.off_carry_base);
+  p.carry = a->carry;
+  p.prefix = (float*)(ws + L.off_prefix);
+  p.carry_head_stride = L.carry_slots_per_head;
+  p.num_heads = a->num_heads;
+  p.head_dim = a->head_dim;
+  p.scale_log2 = (float)((double)a->logit_scale * kLog2e);
+  p.logit_scale = a->logit_scale;
+  p.attend_current = a->attend_current ? 1 : 0;
+  bool v16 = (a->head_dim % (16 / (int)es)) == 0;
+  for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
+    if (t->ptr) v16 = v16 && vec16(*t, es, fixed);
+  p.vec_ok = v16 ? 1 : 0;
+  if (a->dtype == SBA_F32)
+    return sba::launch_bwd_f32(p, (int)L.max_q_tiles, (int)L.max_k_tiles, stream) == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
+  if (sba::launch_bwd_dq(p, a->dtype == SBA_F16, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  if (sba::launch_bwd_dkv(p, a->dtype == SBA_F16, (int)L.max_k_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  return SBA_OK;
+}
+
+}  // extern "C"

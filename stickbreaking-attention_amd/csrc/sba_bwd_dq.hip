@@ -1,0 +1,157 @@
+// Backward, kernel 1 of 2: dQ, plus the per-(row, key tile) prefix sums that make the dK/dV kernel lock-free.
+//
+// One workgroup per tile of 128 query rows (wave w owns rows 32w..32w+31, lane l owns query l%32), key tiles
+// of 64 swept FORWARDS from key 0 to the diagonal.  With g_ij = A_ij (dO_i.v_j - drem_i) the logit gradient is
+//     dz_ij = g_ij - sigma_ij * C_ij,     C_ij = sum_{j' <= j} g_ij'        (sb_varlen_bwd.py:438-447)
+// so C is a running prefix sum in this direction and needs no anchor.  (sigma does not decay with distance, so
+// any constant error in C would be multiplied into every key of the row; C has to be built from exactly the g
+// values it sums.)  A_ij needs the product of (1 - sigma) over the keys ABOVE j instead.  The reference gets
+// it by subtracting a running log-sum from the saved row total (sb_varlen_fwd.py:52-53), which cancels badly
+// on long rows with saturated logits; here the forward, which sweeps downwards from the diagonal, has
+// recorded that product at every tile boundary, and the scan inside a tile runs downwards in registers.
+//
+// Before each key tile J the kernel records C just below J for every row: together with the forward's
+// products the key-stationary dK/dV kernel can start its per-tile scans from these, so no tile of dK or dV
+// is ever accumulated by more than one workgroup (the reference serialises that accumulation behind a spin
+// lock per key tile: sb_varlen_bwd.py:11-53).
+#include "sba_device.hpp"
+#include "sba_params.hpp"
+
+namespace sba {
+
+template <typename T, int DH>
+__global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
+  typedef typename Elem<T>::vec8 vec8;
+  constexpr int kRowStride = DH + kPad;
+  constexpr int kSteps = DH / 16;
+  constexpr int kDTiles = DH / 32;
+  __shared__ __attribute__((aligned(16))) T k_lds[kBlockK * kRowStride];
+  __shared__ __attribute__((aligned(16))) T v_lds[kBlockK * kRowStride];
+
+  int head, slot;
+  xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
+  if (slot >= p.counts[0]) return;
+  const Tile tile = p.q_tiles[slot];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, col = lane & 31;
+  const int L = tile.seq_len, q0 = tile.origin, ac = p.attend_current, D = p.head_dim;
+  const bool vec_ok = p.vec_ok != 0;
+  const int64_t tok0 = tile.seq_start;
+
+  const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
+  const T* kb = (const T*)p.k.ptr + tile.seq_id * p.k.sb + head * p.k.sh + tok0 * p.k.st;
+  const T* vb = (const T*)p.v.ptr + tile.seq_id * p.v.sb + head * p.v.sh + tok0 * p.v.st;
+  const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
+
+  const int qi = q0 + wave * 32 + col;
+  const bool row_ok = qi < L;
+  vec8 qf[kSteps], dof[kSteps];
+#pragma unroll
+  for (int kk = 0; kk < kSteps; kk++) {
+    const int d0 = 16 * kk + 8 * half;
+    qf[kk] = as_vec8<T>(load_row8<T>(qb + (int64_t)qi * p.q.st, d0, D, row_ok, vec_ok));
+    dof[kk] = as_vec8<T>(load_row8<T>(dob + (int64_t)qi * p.d_o.st, d0, D, row_ok, vec_ok));
+  }
+  float drem = 0.f;
+  if (row_ok && p.d_rem.ptr)
+    drem = (float)((const T*)p.d_rem.ptr)[tile.seq_id * p.d_rem.sb + head * p.d_rem.sh + (tok0 + qi) * p.d_rem.st];
+  float prefix = 0.f;      // sum of g over the keys already swept (both half-waves hold the same value)
+
+  const int last_row = min(q0 + kBlockQ, L) - 1;
+  const int last_key = last_row - 1 + ac;
+  const int n_kt = last_key < 0 ? 0 : last_key / kBlockK + 1;
+  const int w_first = q0 + wave * 32, w_last = w_first + 31;
+  const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
+  const int64_t slot0 = (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id];
+  const float* carry = p.carry + slot0;
+  float* prefix_out = p.prefix + slot0;
+
+  f32x16 dqacc[kDTiles];
+#pragma unroll
+  for (int dt = 0; dt < kDTiles; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dqacc[dt][r] = 0.f;
+
+  TileCopy<T, DH, kBlockK> ck, cv;
+  if (n_kt > 0) {
+    ck.load(kb, p.k.st, L, D, vec_ok);
+    cv.load(vb, p.v.st, L, D, vec_ok);
+  }
+  for (int jt = 0; jt < n_kt; ++jt) {
+    const int j0 = jt * kBlockK;
+    __syncthreads();
+    ck.store(k_lds);
+    cv.store(v_lds);
+    __syncthreads();
+    if (jt + 1 < n_kt) {
+      const int jn = j0 + kBlockK;
+      ck.load(kb + (int64_t)jn * p.k.st, p.k.st, L - jn, D, vec_ok);
+      cv.load(vb + (int64_t)jn * p.v.st, p.v.st, L - jn, D, vec_ok);
+    }
+    // For the key-stationary kernel: C just below this tile, for every row of the tile.
+    const int64_t slot_idx = carry_offset(jt, n_qt) + (qi - kBlockQ * (jt >> 1));
+    if (half == 0) prefix_out[slot_idx] = prefix;
+    if (j0 > w_last - 1 + ac) continue;
+    const bool diagonal = (j0 + kBlockK - 1) > (w_first - 1 + ac) || w_last >= L;
+
+    f32x16 s[2], dp[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) { s[mt][r] = 0.f; dp[mt][r] = 0.f; }
+      const int krow = mfma_row_to_key(mt, col);
+#pragma unroll
+      for (int kk = 0; kk < kSteps; kk++) {
+        vec8 a = lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half);
+        s[mt] = Elem<T>::mfma(a, qf[kk], s[mt]);
+      }
+#pragma unroll
+      for (int kk = 0; kk < kSteps; kk++) {
+        vec8 a = lds_row8<T>(v_lds, kRowStride, krow, 16 * kk + 8 * half);
+        dp[mt] = Elem<T>::mfma(a, dof[kk], dp[mt]);
+      }
+    }
+    const int lim = row_ok ? qi + ac - j0 - 32 * half : 0;
+    uint32_t pk[16], dzk[16];
+    bwd_tile_math<T>(s, dp, p.scale_log2, diagonal, lim, half, drem, carry[slot_idx], prefix, pk, dzk, prefix);
+
+    // dQ += dZ K: A = dZ from registers, B = K gathered down the keys.
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      u32x4 av = {dzk[4 * c], dzk[4 * c + 1], dzk[4 * c + 2], dzk[4 * c + 3]};
+      vec8 a = as_vec8<T>(av);
+#pragma unroll
+      for (int dt = 0; dt < kDTiles; dt++) {
+        vec8 b = lds_col8<T>(k_lds, kRowStride, 32 * half + 8 * c, 32 * dt, lane);
+        dqacc[dt] = Elem<T>::mfma(a, b, dqacc[dt]);
+      }
+    }
+  }
+
+  T* dqb = (T*)p.dq.ptr + tile.seq_id * p.dq.sb + head * p.dq.sh + tok0 * p.dq.st;
+#pragma unroll
+  for (int dt = 0; dt < kDTiles; dt++) {
+    const int d = 32 * dt + col;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int row = w_first + 8 * (r >> 2) + 4 * half + (r & 3);
+      if (row < L && d < D) dqb[(int64_t)row * p.dq.st + d] = (T)(dqacc[dt][r] * p.logit_scale);
+    }
+  }
+}
+
+template <typename T>
+static hipError_t launch_t(const BwdParams& p, int max_tiles, hipStream_t stream) {
+  const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kThreads);
+  if (p.head_dim <= 64) {
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 64>), grid, block, 0, stream, p);
+  } else {
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 128>), grid, block, 0, stream, p);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_bwd_dq(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream) {
+  return dtype_is_f16 ? launch_t<_Float16>(p, max_tiles, stream) : launch_t<__bf16>(p, max_tiles, stream);
+}
+
+}  // namespace sba

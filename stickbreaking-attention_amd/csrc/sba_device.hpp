@@ -1,0 +1,246 @@
+// Device-side building blocks shared by the gfx950 stick-breaking attention kernels.
+//
+// Register-level conventions used everywhere in this library
+// ----------------------------------------------------------
+// Scores are produced TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16_{bf16,f16}: the 32 MFMA rows
+// are keys, the 32 MFMA columns are queries.  In the 32x32 accumulator lane l holds column l%32 and
+// the 16 rows 8*(r/4) + 4*(l/32) + r%4 (r = register index).  The key <-> MFMA-row assignment is free
+// (it only decides which LDS row a lane fetches for the A operand), and it is chosen so that for a
+// key tile of 64 keys (two MFMA row tiles mt = 0, 1) lane l owns query l%32 and the 32 CONSECUTIVE
+// keys 32*(l/32) + 16*mt + r.  The stick-breaking products along the key axis are then serial
+// in-register scans with a single exchange between the two half-waves per tile, and the registers
+// feed the next MFMA (P.V, dZ.K) directly as its A operand (k index = 8*(l/32) + t  <->  key
+// 32*(l/32) + 8*c + t for k-step c).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "sba_params.hpp"
+
+namespace sba {
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+constexpr int kBlockQ = 128;   // query rows per workgroup tile (4 waves x 32)
+constexpr int kBlockK = 64;    // keys per tile
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+
+// Element-type traits: 16-bit storage types with an MFMA 32x32x16 variant.
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+  typedef bf16x8 vec8;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Elem<_Float16> {
+  typedef f16x8 vec8;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// Two fp32 -> packed 16-bit (round to nearest even), low half = a.
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2<__bf16>(float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  bf16x2 v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+template <> __device__ __forceinline__ uint32_t pack2<_Float16>(float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+  f16x2 v = {(_Float16)a, (_Float16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
+
+template <typename T> __device__ __forceinline__ typename Elem<T>::vec8 as_vec8(u32x4 x) {
+  return __builtin_bit_cast(typename Elem<T>::vec8, x);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }   // v_exp_f32
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }    // v_log_f32
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }     // v_rcp_f32
+__device__ __forceinline__ float fast_min(float a, float b) {
+  float r;
+  asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// Value held by the other half-wave (lane ^ 32).
+__device__ __forceinline__ float other_half(float x, int half) {
+  uint32_t u = __builtin_bit_cast(uint32_t, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  // r[0]: low lanes keep their own value, high lanes receive lane-32's; r[1]: low lanes receive lane+32's.
+  uint32_t o = half ? r[0] : r[1];
+  return __builtin_bit_cast(float, o);
+}
+
+// LDS row-major tile of 16-bit elements with `kPad` elements of padding per row.
+constexpr int kPad = 8;
+
+// 8 consecutive elements of one row (A operand for contractions over head_dim, or over a row's own axis).
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::vec8 lds_row8(const T* tile, int row_stride, int row, int col) {
+  return *reinterpret_cast<const typename Elem<T>::vec8*>(tile + row * row_stride + col);
+}
+
+// B operand gathered DOWN the rows of a row-major tile with the gfx950 LDS transpose read:
+// returns, for this lane's column `col0 + l%32`, the 8 elements of rows row0 .. row0+7.
+// Within each 16-lane group, lane s fetches the 8-byte chunk (row row0 + 4*t + s/4, columns
+// cbase + 4*(s%4) .. +3) and receives rows row0+4*t .. +3 of column cbase + s.
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::vec8 lds_col8(const T* tile, int row_stride, int row0, int col0, int lane) {
+  const int s = lane & 15;
+  const int cbase = col0 + ((lane >> 4) & 1) * 16;
+  const T* p0 = tile + (row0 + (s >> 2)) * row_stride + cbase + 4 * (s & 3);
+  const T* p1 = p0 + 4 * row_stride;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p1));
+  typedef __attribute__((ext_vector_type(8))) short s16x8;
+  s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(typename Elem<T>::vec8, v);
+}
+
+// MFMA row m (A-operand lane index l%32) of row tile mt -> key offset inside the 64-key tile such that
+// accumulator register r of half-wave h holds key 32*h + 16*mt + r.  (m = 8a + 4h + b, r = 4a + b.)
+__device__ __forceinline__ int mfma_row_to_key(int mt, int m) {
+  return ((m >> 2) & 1) * 32 + mt * 16 + (m >> 3) * 4 + (m & 3);
+}
+
+// Cooperative global -> register -> LDS copy of a [kRows x DH] tile of 16-bit elements, 16 bytes per access.
+// Rows at or beyond `rows_valid` and columns at or beyond `d_valid` are zero-filled.
+template <typename T, int DH, int kRows>
+struct TileCopy {
+  static constexpr int kChunksPerRow = DH / 8;
+  static constexpr int kChunks = kRows * kChunksPerRow;
+  static constexpr int kPerThread = kChunks / kThreads;
+  static_assert(kChunks % kThreads == 0, "tile must divide evenly over the workgroup");
+  u32x4 regs[kPerThread];
+
+  __device__ __forceinline__ void load(const T* base, int64_t row_stride, int rows_valid, int d_valid, bool vec_ok) {
+#pragma unroll
+    for (int i = 0; i < kPerThread; i++) {
+      const int c = threadIdx.x + i * kThreads;
+      const int row = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
+      u32x4 v = {0, 0, 0, 0};
+      if (row < rows_valid) {
+        const T* p = base + row * row_stride + col;
+        if (vec_ok && col + 8 <= d_valid) {
+          v = *reinterpret_cast<const u32x4*>(p);
+        } else {
+          uint16_t e[8];
+#pragma unroll
+          for (int t = 0; t < 8; t++) e[t] = (col + t < d_valid) ? reinterpret_cast<const uint16_t*>(p)[t] : (uint16_t)0;
+          v[0] = e[0] | ((uint32_t)e[1] << 16); v[1] = e[2] | ((uint32_t)e[3] << 16);
+          v[2] = e[4] | ((uint32_t)e[5] << 16); v[3] = e[6] | ((uint32_t)e[7] << 16);
+        }
+      }
+      regs[i] = v;
+    }
+  }
+  __device__ __forceinline__ void store(T* tile) const {
+#pragma unroll
+    for (int i = 0; i < kPerThread; i++) {
+      const int c = threadIdx.x + i * kThreads;
+      const int row = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
+      *reinterpret_cast<u32x4*>(tile + row * (DH + kPad) + col) = regs[i];
+    }
+  }
+};
+
+// Load 8 consecutive head_dim elements of one token row from global memory (zero beyond head_dim / when !valid).
+template <typename T>
+__device__ __forceinline__ u32x4 load_row8(const T* row, int d0, int d_valid, bool valid, bool vec_ok) {
+  u32x4 v = {0, 0, 0, 0};
+  if (valid) {
+    if (vec_ok && d0 + 8 <= d_valid) {
+      v = *reinterpret_cast<const u32x4*>(row + d0);
+    } else {
+      uint16_t e[8];
+#pragma unroll
+      for (int t = 0; t < 8; t++) e[t] = (d0 + t < d_valid) ? reinterpret_cast<const uint16_t*>(row + d0)[t] : (uint16_t)0;
+      v[0] = e[0] | ((uint32_t)e[1] << 16); v[1] = e[2] | ((uint32_t)e[3] << 16);
+      v[2] = e[4] | ((uint32_t)e[5] << 16); v[3] = e[6] | ((uint32_t)e[7] << 16);
+    }
+  }
+  return v;
+}
+
+constexpr float kExpClamp = 100.0f;   // 2^100 and 2^-100 are finite; sigma(z) is 1 - 2^-100 there
+
+// Element-wise backward math of one 64-key tile for the 32 keys this lane owns (see the conventions above).
+//   s, dp     : S^T = K Q^T and dP^T = V dO^T accumulators (row tile mt, register r  <->  key 32*half + 16*mt + r)
+//   lim       : key R of this lane is visible iff R < lim (only consulted when `diagonal`)
+//   prod_in   : prod over the keys ABOVE this tile (between the tile and the row) of (1 - sigma); recorded by
+//               the forward, which sweeps in that direction
+//   prefix_in : sum over the keys BELOW this tile of g, with g_ij = A_ij (dO_i.v_j - drem_i)
+// Produces P (pk) and dZ = g - sigma * C (dzk), C_ij = sum_{j' <= j} g_ij', packed to 16 bit two keys per
+// word, and the prefix sum for the next tile up.  (The reference evaluates the same quantities tile by tile at
+// stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:438-447.)
+template <typename T>
+__device__ __forceinline__ void bwd_tile_math(const f32x16 (&s)[2], const f32x16 (&dp)[2], float scale_log2, bool diagonal,
+                                              int lim, int half, float drem, float prod_in, float prefix_in,
+                                              uint32_t (&pk)[16], uint32_t (&dzk)[16], float& prefix_out) {
+  float beta[32], pr[32], cum[32];
+  float run = 1.f;
+#pragma unroll
+  for (int R = 31; R >= 0; --R) {
+    float x = s[R >> 4][R & 15] * scale_log2;
+    x = fast_min(x, kExpClamp);
+    if (diagonal) x = (R < lim) ? x : -INFINITY;
+    const float e = fast_exp2(x);
+    const float omb = fast_rcp(1.f + e);
+    beta[R] = e * omb;
+    pr[R] = run;           // product over this lane's higher keys
+    run *= omb;
+  }
+  const float oth = other_half(run, half);
+  const float seed = half ? prod_in : prod_in * oth;      // the upper half-wave holds the higher keys
+  float acc = 0.f;
+#pragma unroll
+  for (int R = 0; R < 32; R++) {
+    const float a = beta[R] * (pr[R] * seed);
+    pr[R] = a;
+    acc += a * (dp[R >> 4][R & 15] - drem);
+    cum[R] = acc;          // inclusive prefix sum of g over this lane's keys
+  }
+  const float oth_g = other_half(acc, half);
+  const float base = half ? prefix_in + oth_g : prefix_in;  // the lower half-wave holds the lower keys
+  prefix_out = prefix_in + (acc + oth_g);
+#pragma unroll
+  for (int R = 0; R < 32; R += 2) {
+    const float g0 = cum[R] - (R ? cum[R - 1] : 0.f);
+    const float g1 = cum[R + 1] - cum[R];
+    const float dz0 = g0 - beta[R] * (base + cum[R]);
+    const float dz1 = g1 - beta[R + 1] * (base + cum[R + 1]);
+    pk[R >> 1] = pack2<T>(pr[R], pr[R + 1]);
+    dzk[R >> 1] = pack2<T>(dz0, dz1);
+  }
+}
+
+// Map the linear workgroup id to (head, tile slot) so that the workgroups of one head land on one XCD
+// (workgroups are dealt round-robin to the 8 XCDs, each with a private L2): K/V of a head are then
+// re-read from that XCD's L2 rather than from HBM.
+__device__ __forceinline__ void xcd_head_tile(int wg, int num_heads, int* head, int* slot) {
+  if ((num_heads & 7) == 0) {
+    const int hpx = num_heads >> 3;
+    const int xcd = wg & 7, r = wg >> 3;
+    *head = xcd * hpx + (r % hpx);
+    *slot = r / hpx;
+  } else {
+    *head = wg % num_heads;
+    *slot = wg / num_heads;
+  }
+}
+
+}  // namespace sba

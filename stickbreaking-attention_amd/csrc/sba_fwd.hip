@@ -1,0 +1,172 @@
+// Forward stick-breaking attention for gfx950.
+//
+// One workgroup = one tile of 128 query rows of one (head, sequence); wave w owns rows 32w..32w+31, lane l
+// owns query l%32.  Key tiles of 64 keys are swept in REVERSE from the causal diagonal (the order in which
+// the stick is broken: stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:155-165), so the running product
+// prod_{j<k<i} (1 - sigma(z_ik)) is carried forward in registers and never has to be divided out.
+//
+// Per element, in linear space (base-2 exponentials, as sb_varlen_fwd.py:296 and softplus.py:8-12 do):
+//     e = 2^x, x = z log2(e)          1 - sigma = 1/(1+e)          sigma = e/(1+e)
+//     A_ij = e_ij * prod_{j<=k<i} 1/(1+e_ik)
+// which needs two transcendentals (v_exp_f32, v_rcp_f32) where the log-space form
+// log A = x - softplus2(x) + cumsum(-softplus2) needs three.  The product can only underflow where A itself is
+// below 2^-126, and row_stat = log2(prod) is taken once per row at the end.
+#include "sba_device.hpp"
+#include "sba_params.hpp"
+
+namespace sba {
+
+template <typename T, int DH>
+__global__ __launch_bounds__(kThreads) void fwd_kernel(FwdParams p) {
+  typedef typename Elem<T>::vec8 vec8;
+  constexpr int kRowStride = DH + kPad;
+  constexpr int kSteps = DH / 16;    // MFMA k-steps over head_dim
+  constexpr int kDTiles = DH / 32;   // 32-wide output tiles over head_dim
+  __shared__ __attribute__((aligned(16))) T k_lds[kBlockK * kRowStride];
+  __shared__ __attribute__((aligned(16))) T v_lds[kBlockK * kRowStride];
+
+  int head, slot;
+  xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
+  if (slot >= p.counts[0]) return;
+  const Tile tile = p.tiles[slot];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, col = lane & 31;
+  const int L = tile.seq_len, q0 = tile.origin, ac = p.attend_current, D = p.head_dim;
+  const bool vec_ok = p.vec_ok != 0;
+
+  const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + (int64_t)tile.seq_start * p.q.st;
+  const T* kb = (const T*)p.k.ptr + tile.seq_id * p.k.sb + head * p.k.sh + (int64_t)tile.seq_start * p.k.st;
+  const T* vb = (const T*)p.v.ptr + tile.seq_id * p.v.sb + head * p.v.sh + (int64_t)tile.seq_start * p.v.st;
+
+  // This lane's query row as the B operand of S^T = K Q^T: 8 consecutive head_dim elements per k-step.
+  const int qi = q0 + wave * 32 + col;
+  vec8 qf[kSteps];
+#pragma unroll
+  for (int kk = 0; kk < kSteps; kk++)
+    qf[kk] = as_vec8<T>(load_row8<T>(qb + (int64_t)qi * p.q.st, 16 * kk + 8 * half, D, qi < L, vec_ok));
+
+  const int last_row = min(q0 + kBlockQ, L) - 1;
+  const int last_key = last_row - 1 + ac;                    // last key any row of this tile can see
+  const int n_kt = last_key < 0 ? 0 : last_key / kBlockK + 1;
+  const int w_first = q0 + wave * 32, w_last = w_first + 31;   // this wave's rows
+
+  f32x16 oacc[kDTiles];
+#pragma unroll
+  for (int dt = 0; dt < kDTiles; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) oacc[dt][r] = 0.f;
+  float prod = 1.f;    // prod over the keys already swept of (1 - sigma): both half-waves hold the same value
+  const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
+  float* carry = p.carry ? p.carry + (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] : nullptr;
+
+  TileCopy<T, DH, kBlockK> ck, cv;
+  if (n_kt > 0) {
+    const int j0 = (n_kt - 1) * kBlockK;
+    ck.load(kb + (int64_t)j0 * p.k.st, p.k.st, L - j0, D, vec_ok);
+    cv.load(vb + (int64_t)j0 * p.v.st, p.v.st, L - j0, D, vec_ok);
+  }
+  for (int jt = n_kt - 1; jt >= 0; --jt) {
+    const int j0 = jt * kBlockK;
+    __syncthreads();
+    ck.store(k_lds);
+    cv.store(v_lds);
+    __syncthreads();
+    if (jt > 0) {
+      const int jn = j0 - kBlockK;
+      ck.load(kb + (int64_t)jn * p.k.st, p.k.st, L - jn, D, vec_ok);
+      cv.load(vb + (int64_t)jn * p.v.st, p.v.st, L - jn, D, vec_ok);
+    }
+    // For the backward: the product over the keys between this tile and the row, for every row of the tile.
+    if (carry && half == 0) carry[carry_offset(jt, n_qt) + (qi - kBlockQ * (jt >> 1))] = prod;
+    if (j0 > w_last - 1 + ac) continue;                       // nothing visible to this wave yet
+    const bool diagonal = (j0 + kBlockK - 1) > (w_first - 1 + ac);
+
+    // S^T tile: rows = keys (permuted so that a lane ends up with 32 consecutive keys), columns = queries.
+    f32x16 s[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) s[mt][r] = 0.f;
+      const int krow = mfma_row_to_key(mt, col);
+#pragma unroll
+      for (int kk = 0; kk < kSteps; kk++) {
+        vec8 a = lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half);
+        s[mt] = Elem<T>::mfma(a, qf[kk], s[mt]);
+      }
+    }
+
+    // e = 2^x for this lane's 32 keys j0 + 32*half + R, R = 16*mt + r; hidden keys get e = 0 (factor 1, weight 0).
+    float e[32];
+    const int lim = qi + ac - j0 - 32 * half;                 // key R is visible iff R < lim
+#pragma unroll
+    for (int R = 0; R < 32; R++) {
+      float x = s[R >> 4][R & 15] * p.scale_log2;
+      x = fast_min(x, kExpClamp);
+      if (diagonal) x = (R < lim) ? x : -INFINITY;
+      e[R] = fast_exp2(x);
+    }
+    // w[R] = prod_{R' >= R} 1/(1+e[R'])  (reverse inclusive scan along this lane's keys)
+    float w[32];
+    float run = 1.f;
+#pragma unroll
+    for (int R = 31; R >= 0; --R) {
+      const float omb = fast_rcp(1.f + e[R]);
+      run = (R == 31) ? omb : run * omb;
+      w[R] = run;
+    }
+    const float oth = other_half(run, half);
+    // The upper half-wave holds the higher keys, which come first in the sweep.
+    const float seed = half ? prod : prod * oth;
+    prod = (prod * oth) * run;
+
+    uint32_t pk[16];
+#pragma unroll
+    for (int R = 0; R < 32; R += 2) pk[R >> 1] = pack2<T>(e[R] * (w[R] * seed), e[R + 1] * (w[R + 1] * seed));
+
+    // O += P V: A = P from registers (k index <-> key 32*half + 8c + t), B = V gathered down the keys.
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      u32x4 av = {pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
+      vec8 a = as_vec8<T>(av);
+#pragma unroll
+      for (int dt = 0; dt < kDTiles; dt++) {
+        vec8 b = lds_col8<T>(v_lds, kRowStride, 32 * half + 8 * c, 32 * dt, lane);
+        oacc[dt] = Elem<T>::mfma(a, b, oacc[dt]);
+      }
+    }
+  }
+
+  // Epilogue.  oacc[dt][r]: query row 8*(r/4) + 4*half + r%4 of this wave, column 32*dt + col.
+  T* ob = (T*)p.o.ptr + tile.seq_id * p.o.sb + head * p.o.sh + (int64_t)tile.seq_start * p.o.st;
+#pragma unroll
+  for (int dt = 0; dt < kDTiles; dt++) {
+    const int d = 32 * dt + col;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int row = w_first + 8 * (r >> 2) + 4 * half + (r & 3);
+      if (row < L && d < D) ob[(int64_t)row * p.o.st + d] = (T)oacc[dt][r];
+    }
+  }
+  if (half == 0 && qi < L) {
+    T* rb = (T*)p.rem.ptr + tile.seq_id * p.rem.sb + head * p.rem.sh + (int64_t)(tile.seq_start + qi) * p.rem.st;
+    *rb = (T)prod;
+    p.row_stat[tile.seq_id * p.stat_sb + head * p.stat_sh + tile.seq_start + qi] = fast_log2(prod);
+  }
+}
+
+template <typename T>
+static hipError_t launch_fwd_t(const FwdParams& p, int dh, int max_tiles, hipStream_t stream) {
+  const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kThreads);
+  if (dh <= 64) {
+    hipLaunchKernelGGL((fwd_kernel<T, 64>), grid, block, 0, stream, p);
+  } else {
+    hipLaunchKernelGGL((fwd_kernel<T, 128>), grid, block, 0, stream, p);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_fwd(const FwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream) {
+  return dtype_is_f16 ? launch_fwd_t<_Float16>(p, p.head_dim, max_tiles, stream)
+                      : launch_fwd_t<__bf16>(p, p.head_dim, max_tiles, stream);
+}
+
+}  // namespace sba

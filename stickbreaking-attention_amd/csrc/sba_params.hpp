@@ -1,0 +1,81 @@
+// Kernel parameter blocks shared by the host launcher and the device code.
+#pragma once
+#include <stdint.h>
+
+namespace sba {
+
+struct TensorRef {     // [batch,] head, token, head_dim; element strides; head_dim stride 1
+  void* ptr;
+  int64_t sb, sh, st;
+};
+struct VectorRef {     // [batch,] head, token
+  void* ptr;
+  int64_t sb, sh, st;
+};
+
+// Tile descriptor produced by the scheduler kernel.
+struct Tile {
+  int32_t seq_start;   // first token of the sequence in the packed token axis (0 in fixed-length mode)
+  int32_t seq_len;
+  int32_t origin;      // first query row (query tiles) or first key (key tiles), relative to the sequence
+  int32_t seq_id;      // sequence index; selects the batch stride in fixed-length mode
+};
+
+struct SchedParams {
+  const void* cu;          // NULL: fixed-length mode
+  int32_t cu_is_int64, cu_has_leading_zero;
+  int32_t num_seqs;
+  int32_t fixed_len;       // L in fixed-length mode
+  int32_t attend_current;
+  int32_t want_key_tiles;  // backward: also build the key-tile list
+  int32_t want_carry_base; // also lay out the per-sequence carry offsets
+  Tile* q_tiles;           // query tiles (kBlockQ rows), heaviest first
+  Tile* k_tiles;           // key tiles (kBlockK keys), heaviest first
+  int32_t* counts;         // [0] = number of query tiles, [1] = number of key tiles
+  int64_t* carry_base;     // per sequence: first carry slot of the sequence (per head)
+};
+
+struct FwdParams {
+  TensorRef q, k, v, o;
+  VectorRef rem;
+  float* row_stat;
+  int64_t stat_sb, stat_sh;    // row_stat strides (token stride 1)
+  float* carry;                // optional [head][slot]: running product per (row, key tile)
+  const int64_t* carry_base;
+  int64_t carry_head_stride;
+  const Tile* tiles;
+  const int32_t* counts;
+  int32_t num_heads, head_dim;
+  float scale_log2;            // logit_scale * log2(e)
+  int32_t attend_current;
+  int32_t vec_ok;              // all row strides / base pointers allow 16-byte accesses and head_dim % 8 == 0
+};
+
+struct BwdParams {
+  TensorRef q, k, v, d_o, dq, dk, dv;
+  VectorRef d_rem;
+  const Tile* q_tiles;
+  const Tile* k_tiles;
+  const int32_t* counts;
+  const int64_t* carry_base;
+  const float* carry;          // [head][slot]: the forward's running product per (row, key tile)
+  float* prefix;               // [head][slot]: prefix sum of g over the keys below the tile, per (row, key tile)
+  int64_t carry_head_stride;   // carry slots reserved per head
+  int32_t num_heads, head_dim;
+  float scale_log2;
+  float logit_scale;
+  int32_t attend_current;
+  int32_t vec_ok;
+};
+
+// Carry slots of one sequence whose length rounds up to M query tiles: key tiles 2m and 2m+1 are needed
+// by the rows of query tiles m, m+1, ..., M-1.  Slot of (key tile J, row i), i >= 128*(J/2):
+//   carry_offset(J, M) + (i - 128*(J/2))
+__host__ __device__ inline int64_t carry_offset(int64_t J, int64_t M) {
+  const int64_t m = J >> 1;
+  const int64_t tri = (J & 1) ? m * m : m * (m - 1);      // sum_{J' < J} floor(J'/2)
+  return J * (M * 128) - 128 * tri;
+}
+__host__ __device__ inline int64_t carry_slots(int64_t M) { return 128 * M * (M + 1); }   // carry_offset(2M, M)
+
+}  // namespace sba

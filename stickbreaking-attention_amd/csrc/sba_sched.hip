@@ -1,0 +1,145 @@
+// cu_seqlens -> tile scheduler.
+//
+// The reference pads every sequence to the longest one: its grid is (num_seqs, H/2, max_len/64 + 1) programs,
+// most of which exit idle on a ragged batch (stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:475-479, :294).
+// Here a single small kernel reads cu_seqlens on the device (no host synchronisation), enumerates exactly the
+// tiles that exist and orders them heaviest first (a query tile that starts at row q0 sweeps ~q0/64 key
+// tiles), so the one launch that follows fills the chip without padding and ends with the cheap tiles.
+// It also lays out the backward's per-(row, key tile) carries contiguously per sequence.
+#include "sba_device.hpp"
+#include "sba_params.hpp"
+
+namespace sba {
+
+constexpr int kBins = 4096;          // work histogram bins (work = number of tiles swept, saturating)
+constexpr int kSchedThreads = 1024;
+
+__device__ __forceinline__ int64_t read_cu(const SchedParams& p, int idx) {
+  return p.cu_is_int64 ? ((const int64_t*)p.cu)[idx] : (int64_t)((const int32_t*)p.cu)[idx];
+}
+__device__ __forceinline__ void seq_bounds(const SchedParams& p, int s, int* start, int* len) {
+  if (p.cu == nullptr) { *start = 0; *len = p.fixed_len; return; }
+  const int off = p.cu_has_leading_zero ? 1 : 0;
+  const int64_t end = read_cu(p, s + off);
+  const int64_t beg = (s + off == 0) ? 0 : read_cu(p, s + off - 1);
+  *start = (int)beg;
+  *len = (int)(end > beg ? end - beg : 0);
+}
+// Number of key tiles a query tile sweeps.
+__device__ __forceinline__ int q_tile_work(int q0, int len, int ac) {
+  const int last_key = min(q0 + kBlockQ, len) - 2 + ac;
+  return last_key < 0 ? 0 : last_key / kBlockK + 1;
+}
+// Number of query tiles a key tile is swept by.
+__device__ __forceinline__ int k_tile_work(int j0, int len, int ac) {
+  const int first_row = j0 + 1 - ac;
+  if (first_row >= len) return 0;
+  return (len + kBlockQ - 1) / kBlockQ - first_row / kBlockQ;
+}
+
+// Exclusive prefix sum over bins taken from the heaviest bin downwards; bins[] becomes the start offsets.
+__device__ void descending_offsets(int* bins, int* scratch) {
+  constexpr int kPer = kBins / kSchedThreads;
+  const int t = threadIdx.x;
+  // thread t owns bins (kBins-1 - kPer*t) down to (kBins-1 - kPer*t - kPer + 1)
+  int local[kPer], sum = 0;
+#pragma unroll
+  for (int i = 0; i < kPer; i++) { local[i] = bins[kBins - 1 - (kPer * t + i)]; sum += local[i]; }
+  scratch[t] = sum;
+  __syncthreads();
+  for (int d = 1; d < kSchedThreads; d <<= 1) {
+    const int v = (t >= d) ? scratch[t - d] : 0;
+    __syncthreads();
+    scratch[t] += v;
+    __syncthreads();
+  }
+  int base = scratch[t] - sum;
+#pragma unroll
+  for (int i = 0; i < kPer; i++) { bins[kBins - 1 - (kPer * t + i)] = base; base += local[i]; }
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
+  __shared__ int qbins[kBins];
+  __shared__ int kbins[kBins];
+  __shared__ int scratch[kSchedThreads];
+  __shared__ long long carry_run;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = kSchedThreads / 64;
+  for (int i = threadIdx.x; i < kBins; i += kSchedThreads) { qbins[i] = 0; kbins[i] = 0; }
+  if (threadIdx.x == 0) carry_run = 0;
+  __syncthreads();
+
+  // Pass 1: histogram of tile work.  One wave per sequence, lanes stride over its tiles.
+  for (int s = wave; s < p.num_seqs; s += nwaves) {
+    int start, len;
+    seq_bounds(p, s, &start, &len);
+    const int nq = (len + kBlockQ - 1) / kBlockQ;
+    for (int t = lane; t < nq; t += 64) atomicAdd(&qbins[min(q_tile_work(t * kBlockQ, len, p.attend_current), kBins - 1)], 1);
+    if (p.want_key_tiles) {
+      const int nk = (len + kBlockK - 1) / kBlockK;
+      for (int t = lane; t < nk; t += 64) atomicAdd(&kbins[min(k_tile_work(t * kBlockK, len, p.attend_current), kBins - 1)], 1);
+    }
+  }
+  __syncthreads();
+  descending_offsets(qbins, scratch);
+  if (p.want_key_tiles) descending_offsets(kbins, scratch);
+
+  // Pass 2: scatter the descriptors.
+  for (int s = wave; s < p.num_seqs; s += nwaves) {
+    int start, len;
+    seq_bounds(p, s, &start, &len);
+    const int nq = (len + kBlockQ - 1) / kBlockQ;
+    for (int t = lane; t < nq; t += 64) {
+      const int pos = atomicAdd(&qbins[min(q_tile_work(t * kBlockQ, len, p.attend_current), kBins - 1)], 1);
+      Tile d; d.seq_start = start; d.seq_len = len; d.origin = t * kBlockQ; d.seq_id = s;
+      p.q_tiles[pos] = d;
+    }
+    if (p.want_key_tiles) {
+      const int nk = (len + kBlockK - 1) / kBlockK;
+      for (int t = lane; t < nk; t += 64) {
+        const int pos = atomicAdd(&kbins[min(k_tile_work(t * kBlockK, len, p.attend_current), kBins - 1)], 1);
+        Tile d; d.seq_start = start; d.seq_len = len; d.origin = t * kBlockK; d.seq_id = s;
+        p.k_tiles[pos] = d;
+      }
+    }
+  }
+  __syncthreads();
+  // After the scatter, the lightest bin (work 0) ends at the total count.
+  if (threadIdx.x == 0) {
+    p.counts[0] = qbins[0];
+    p.counts[1] = p.want_key_tiles ? kbins[0] : 0;
+  }
+
+  // Carry layout: exclusive prefix sum of carry_slots(M_s) over sequences (block-wide, chunked).
+  if (p.want_carry_base) {
+    for (int s0 = 0; s0 < p.num_seqs; s0 += kSchedThreads) {
+      const int s = s0 + threadIdx.x;
+      int start = 0, len = 0;
+      if (s < p.num_seqs) seq_bounds(p, s, &start, &len);
+      const long long mine = carry_slots((len + kBlockQ - 1) / kBlockQ);
+      // inclusive scan of `mine` through 64-bit shuffles would need two passes; sequences per chunk are
+      // few enough for a shared-memory Hillis-Steele scan on the low/high words kept as long long.
+      __shared__ long long sc[kSchedThreads];
+      sc[threadIdx.x] = mine;
+      __syncthreads();
+      for (int d = 1; d < kSchedThreads; d <<= 1) {
+        const long long v = (threadIdx.x >= d) ? sc[threadIdx.x - d] : 0;
+        __syncthreads();
+        sc[threadIdx.x] += v;
+        __syncthreads();
+      }
+      const long long base = carry_run;
+      if (s < p.num_seqs) p.carry_base[s] = base + sc[threadIdx.x] - mine;
+      __syncthreads();
+      if (threadIdx.x == kSchedThreads - 1) carry_run = base + sc[threadIdx.x];
+      __syncthreads();
+    }
+  }
+}
+
+hipError_t launch_sched(const SchedParams& p, hipStream_t stream) {
+  hipLaunchKernelGGL(sched_kernel, dim3(1), dim3(kSchedThreads), 0, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace sba

@@ -1,0 +1,6 @@
+"""Stick-breaking attention for AMD MI355X: the operator API of speedcell4/stickbreaking-attention
+(stickbreaking_attention/__init__.py:1-2) on hand-written gfx950 kernels."""
+from .sb_attn import sb_attn
+from .sb_varlen import sb_attn_varlen
+
+__all__ = ["sb_attn", "sb_attn_varlen"]

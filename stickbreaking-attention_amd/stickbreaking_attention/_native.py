@@ -1,0 +1,179 @@
+"""ctypes binding of libsba.so (the C ABI declared in include/sba.h).
+
+This is the only place that touches the shared library.  There is no fallback: if the library has not
+been built, or a call reports an error, the operators raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_LIB_NAME = "libsba.so"
+_lib = None
+
+SBA_BF16, SBA_F32, SBA_F16 = 0, 1, 2
+_DTYPES = {torch.bfloat16: SBA_BF16, torch.float32: SBA_F32, torch.float16: SBA_F16}
+
+
+class SbaTensor(ctypes.Structure):
+    _fields_ = [("ptr", ctypes.c_void_p), ("stride_batch", ctypes.c_int64), ("stride_head", ctypes.c_int64),
+                ("stride_token", ctypes.c_int64)]
+
+
+class SbaVector(ctypes.Structure):
+    _fields_ = SbaTensor._fields_
+
+
+class SbaArgs(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("num_heads", ctypes.c_int32), ("num_seqs", ctypes.c_int32),
+        ("total_tokens", ctypes.c_int64), ("max_seqlen", ctypes.c_int64),
+        ("logit_scale", ctypes.c_float), ("attend_current", ctypes.c_int32),
+        ("cu_seqlens", ctypes.c_void_p), ("cu_is_int64", ctypes.c_int32), ("cu_has_leading_zero", ctypes.c_int32),
+        ("q", SbaTensor), ("k", SbaTensor), ("v", SbaTensor), ("o", SbaTensor),
+        ("rem", SbaVector), ("row_stat", ctypes.c_void_p), ("carry", ctypes.c_void_p),
+        ("d_o", SbaTensor), ("d_rem", SbaVector), ("dq", SbaTensor), ("dk", SbaTensor), ("dv", SbaTensor),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t), ("stream", ctypes.c_void_p),
+    ]
+
+
+EXPORTS = ("sba_version", "sba_strerror", "sba_workspace_bytes", "sba_fwd", "sba_bwd")
+
+
+def library_path() -> str:
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+
+
+def lib():
+    """Load libsba.so once.  Raises if it has not been built (run `make -C csrc` or __graft_entry__.build())."""
+    global _lib
+    if _lib is None:
+        path = library_path()
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `make -C stickbreaking-attention_amd/csrc`; "
+                               "stick-breaking attention has no fallback path")
+        handle = ctypes.CDLL(path)
+        handle.sba_version.restype = ctypes.c_int
+        handle.sba_strerror.restype = ctypes.c_char_p
+        handle.sba_strerror.argtypes = [ctypes.c_int]
+        handle.sba_workspace_bytes.restype = ctypes.c_int
+        handle.sba_workspace_bytes.argtypes = [ctypes.POINTER(SbaArgs)] + [ctypes.POINTER(ctypes.c_size_t)] * 3
+        for name in ("sba_fwd", "sba_bwd"):
+            fn = getattr(handle, name)
+            fn.restype = ctypes.c_int
+            fn.argtypes = [ctypes.POINTER(SbaArgs)]
+        if handle.sba_version() != 1:
+            raise RuntimeError(f"{path}: ABI version {handle.sba_version()} != 1")
+        _lib = handle
+    return _lib
+
+
+def _check(status: int, what: str):
+    if status != 0:
+        raise RuntimeError(f"{what} failed: {lib().sba_strerror(status).decode()} (status {status})")
+
+
+def _tensor(t: Optional[torch.Tensor], fixed: bool) -> SbaTensor:
+    if t is None:
+        return SbaTensor(None, 0, 0, 0)
+    if fixed:
+        return SbaTensor(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+    return SbaTensor(t.data_ptr(), 0, t.stride(0), t.stride(1))
+
+
+def _vector(t: Optional[torch.Tensor], fixed: bool) -> SbaVector:
+    if t is None:
+        return SbaVector(None, 0, 0, 0)
+    if fixed:
+        return SbaVector(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+    return SbaVector(t.data_ptr(), 0, t.stride(0), t.stride(1))
+
+
+def rows_contiguous(t: torch.Tensor) -> torch.Tensor:
+    """The kernels need unit stride along head_dim (as the reference does, sb_varlen_fwd.py:235)."""
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current) -> SbaArgs:
+    if not q.is_cuda:
+        raise RuntimeError("stick-breaking attention runs on the GPU only (got a CPU tensor)")
+    if q.dtype not in _DTYPES:
+        raise TypeError(f"unsupported dtype {q.dtype}")
+    a = SbaArgs()
+    a.dtype = _DTYPES[q.dtype]
+    fixed = cu_seqlens is None
+    if fixed:
+        B, H, L, D = q.shape
+        a.num_seqs, a.num_heads, a.total_tokens, a.head_dim = B, H, L, D
+        a.cu_seqlens = None
+    else:
+        H, T, D = q.shape
+        a.num_heads, a.total_tokens, a.head_dim = H, T, D
+        a.num_seqs = cu_seqlens.numel() - (1 if cu_has_leading_zero else 0)
+        a.cu_seqlens = cu_seqlens.data_ptr()
+        a.cu_is_int64 = 1 if cu_seqlens.dtype == torch.int64 else 0
+        a.cu_has_leading_zero = 1 if cu_has_leading_zero else 0
+    a.max_seqlen = int(max_seqlen) if max_seqlen else 0
+    a.logit_scale = float(logit_scale)
+    a.attend_current = 1 if attend_current else 0
+    a.stream = torch.cuda.current_stream(q.device).cuda_stream
+    return a
+
+
+def prepare_cu_seqlens(cu_seqlens: torch.Tensor, device) -> torch.Tensor:
+    if cu_seqlens.dtype not in (torch.int32, torch.int64):
+        cu_seqlens = cu_seqlens.to(torch.int64)
+    if cu_seqlens.device != device:
+        cu_seqlens = cu_seqlens.to(device)
+    return cu_seqlens.contiguous()
+
+
+def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, want_carry):
+    """Launch the forward.  Returns (o, rem, row_stat, carry or None).  Packed mode when cu_seqlens is given.
+    ``carry`` is the buffer the backward needs; it is only produced when ``want_carry``."""
+    fixed = cu_seqlens is None
+    q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)
+    with torch.cuda.device(q.device):
+        a = _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current)
+        o = torch.empty_like(q)
+        if o.stride(-1) != 1:
+            o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
+        row_stat = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
+        a.q, a.k, a.v, a.o = (_tensor(t, fixed) for t in (q, k, v, o))
+        a.rem = _vector(rem, fixed)
+        a.row_stat = row_stat.data_ptr()
+        need, need_carry = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        _check(lib().sba_workspace_bytes(ctypes.byref(a), ctypes.byref(need), None, ctypes.byref(need_carry)), "sba_workspace_bytes")
+        ws = torch.empty(need.value, dtype=torch.uint8, device=q.device)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), need.value
+        carry = None
+        if want_carry:
+            carry = torch.empty(need_carry.value // 4, dtype=torch.float32, device=q.device)
+            a.carry = carry.data_ptr()
+        _check(lib().sba_fwd(ctypes.byref(a)), "sba_fwd")
+    return o, rem, row_stat, carry
+
+
+def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current):
+    """Launch the backward.  Returns (dq, dk, dv)."""
+    fixed = cu_seqlens is None
+    do = rows_contiguous(do)
+    q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)
+    with torch.cuda.device(q.device):
+        a = _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        if drem is not None and drem.dtype != q.dtype:
+            drem = drem.to(q.dtype)
+        a.q, a.k, a.v, a.d_o, a.dq, a.dk, a.dv = (_tensor(t, fixed) for t in (q, k, v, do, dq, dk, dv))
+        a.d_rem = _vector(drem, fixed)
+        a.carry = carry.data_ptr()
+        need = ctypes.c_size_t(0)
+        _check(lib().sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(need), None), "sba_workspace_bytes")
+        ws = torch.empty(need.value, dtype=torch.uint8, device=q.device)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), need.value
+        _check(lib().sba_bwd(ctypes.byref(a)), "sba_bwd")
+    return dq, dk, dv
