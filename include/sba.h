@@ -92,6 +92,10 @@ typedef struct SbaArgs {
   void* workspace;             /* device scratch, 256-byte aligned */
   size_t workspace_bytes;
   void* stream;                /* hipStream_t */
+  void** trace_events;         /* optional (NULL = off): hipEvent_t handles the library records on `stream` so a
+                                  caller can time the kernels separately.  sba_fwd records [0] before and [1] after
+                                  the attention kernel (the scheduler kernel runs before [0]); sba_bwd records [0]
+                                  before the dQ kernel, [1] between the dQ and dK/dV kernels and [2] after. */
 } SbaArgs;
 
 /* ABI version of this header (SBA_VERSION) the library was built against. */

@@ -163,9 +163,13 @@ int sba_fwd(const SbaArgs* a) {
   bool v16 = (a->head_dim % (16 / (int)es)) == 0;
   for (const SbaTensor* t : {&a->q, &a->k, &a->v}) v16 = v16 && vec16(*t, es, fixed);
   p.vec_ok = v16 ? 1 : 0;
+  hipEvent_t* ev = (hipEvent_t*)a->trace_events;
+  if (ev && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;
   hipError_t e = (a->dtype == SBA_F32) ? sba::launch_fwd_f32(p, (int)L.max_q_tiles, stream)
                                        : sba::launch_fwd(p, a->dtype == SBA_F16, (int)L.max_q_tiles, stream);
-  return e == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
+  if (e != hipSuccess) return SBA_ERR_LAUNCH;
+  if (ev && hipEventRecord(ev[1], stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  return SBA_OK;
 }
 
 int sba_bwd(const SbaArgs* a) {
@@ -209,10 +213,17 @@ int sba_bwd(const SbaArgs* a) {
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
     if (t->ptr) v16 = v16 && vec16(*t, es, fixed);
   p.vec_ok = v16 ? 1 : 0;
-  if (a->dtype == SBA_F32)
-    return sba::launch_bwd_f32(p, (int)L.max_q_tiles, (int)L.max_k_tiles, stream) == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
+  hipEvent_t* ev = (hipEvent_t*)a->trace_events;
+  if (ev && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  if (a->dtype == SBA_F32) {
+    if (sba::launch_bwd_f32(p, (int)L.max_q_tiles, (int)L.max_k_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
+    if (ev && (hipEventRecord(ev[1], stream) != hipSuccess || hipEventRecord(ev[2], stream) != hipSuccess)) return SBA_ERR_LAUNCH;
+    return SBA_OK;
+  }
   if (sba::launch_bwd_dq(p, a->dtype == SBA_F16, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  if (ev && hipEventRecord(ev[1], stream) != hipSuccess) return SBA_ERR_LAUNCH;
   if (sba::launch_bwd_dkv(p, a->dtype == SBA_F16, (int)L.max_k_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  if (ev && hipEventRecord(ev[2], stream) != hipSuccess) return SBA_ERR_LAUNCH;
   return SBA_OK;
 }
 

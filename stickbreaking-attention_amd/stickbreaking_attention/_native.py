@@ -13,6 +13,8 @@ import torch
 
 _LIB_NAME = "libsba.so"
 _lib = None
+# Optional ctypes array of hipEvent_t handed to the next calls as SbaArgs.trace_events (benchmarks only).
+TRACE_EVENTS = None
 
 SBA_BF16, SBA_F32, SBA_F16 = 0, 1, 2
 _DTYPES = {torch.bfloat16: SBA_BF16, torch.float32: SBA_F32, torch.float16: SBA_F16}
@@ -37,6 +39,7 @@ class SbaArgs(ctypes.Structure):
         ("rem", SbaVector), ("row_stat", ctypes.c_void_p), ("carry", ctypes.c_void_p),
         ("d_o", SbaTensor), ("d_rem", SbaVector), ("dq", SbaTensor), ("dk", SbaTensor), ("dv", SbaTensor),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t), ("stream", ctypes.c_void_p),
+        ("trace_events", ctypes.POINTER(ctypes.c_void_p)),
     ]
 
 
@@ -97,9 +100,13 @@ def rows_contiguous(t: torch.Tensor) -> torch.Tensor:
     return t if t.stride(-1) == 1 else t.contiguous()
 
 
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("stick-breaking attention runs on the GPU only (got a CPU tensor); there is no CPU path")
+
+
 def _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current) -> SbaArgs:
-    if not q.is_cuda:
-        raise RuntimeError("stick-breaking attention runs on the GPU only (got a CPU tensor)")
     if q.dtype not in _DTYPES:
         raise TypeError(f"unsupported dtype {q.dtype}")
     a = SbaArgs()
@@ -120,6 +127,8 @@ def _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, atte
     a.logit_scale = float(logit_scale)
     a.attend_current = 1 if attend_current else 0
     a.stream = torch.cuda.current_stream(q.device).cuda_stream
+    if TRACE_EVENTS is not None:
+        a.trace_events = ctypes.cast(TRACE_EVENTS, ctypes.POINTER(ctypes.c_void_p))
     return a
 
 
@@ -134,6 +143,7 @@ def prepare_cu_seqlens(cu_seqlens: torch.Tensor, device) -> torch.Tensor:
 def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, want_carry):
     """Launch the forward.  Returns (o, rem, row_stat, carry or None).  Packed mode when cu_seqlens is given.
     ``carry`` is the buffer the backward needs; it is only produced when ``want_carry``."""
+    _require_gpu(q, k, v)
     fixed = cu_seqlens is None
     q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)
     with torch.cuda.device(q.device):
@@ -160,6 +170,7 @@ def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, a
 
 def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current):
     """Launch the backward.  Returns (dq, dk, dv)."""
+    _require_gpu(q, k, v, do, drem, carry)
     fixed = cu_seqlens is None
     do = rows_contiguous(do)
     q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)

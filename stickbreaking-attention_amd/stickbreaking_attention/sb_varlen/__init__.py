@@ -41,6 +41,7 @@ def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, zero_st
     cu_seqlens = _native.prepare_cu_seqlens(cu_seqlens, q.device)
     if zero_start:
         assert cu_seqlens[0] == 0          # same check (and host sync) as sb_varlen/__init__.py:71-73
+    _native._require_gpu(q, k, v)
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
     return StickBreakingAttention.apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current, bool(zero_start))

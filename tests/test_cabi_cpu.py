@@ -1,0 +1,125 @@
+"""CPU-side checks of the C-ABI library and the host logic: no kernel is launched here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def native():
+    from stickbreaking_attention import _native
+
+    if not os.path.exists(_native.library_path()):
+        import __graft_entry__
+
+        __graft_entry__.build()
+    return _native
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "sba.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"^\s*(?:const\s+)?(?:int|char\s*\*|const char\s*\*)\s*\**\s*(sba_\w+)\s*\(", text, flags=re.M)
+
+
+def test_library_exports_every_declared_symbol(native):
+    names = declared_functions()
+    assert set(names) == set(native.EXPORTS) == {"sba_version", "sba_strerror", "sba_workspace_bytes", "sba_fwd", "sba_bwd"}
+    lib = native.lib()
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.sba_version() == 1
+    assert lib.sba_strerror(0) == b"ok"
+    for code in range(-8, 0):
+        assert lib.sba_strerror(code) not in (b"ok", b"unknown status")
+    assert lib.sba_strerror(-99) == b"unknown status"
+
+
+def test_struct_layout_matches_header(native, tmp_path):
+    src = tmp_path / "sz.c"
+    src.write_text('#include "sba.h"\n#include <stdio.h>\n#include <stddef.h>\nint main(){printf("%zu %zu %zu %zu %zu %zu\\n", '
+                   "sizeof(SbaArgs), offsetof(SbaArgs,q), offsetof(SbaArgs,carry), offsetof(SbaArgs,d_o), "
+                   "offsetof(SbaArgs,workspace), offsetof(SbaArgs,trace_events));}\n")
+    exe = tmp_path / "sz"
+    import subprocess
+
+    subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
+    got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    A = native.SbaArgs
+    assert got == [ctypes.sizeof(A), A.q.offset, A.carry.offset, A.d_o.offset, A.workspace.offset, A.trace_events.offset]
+
+
+def _args(native, H, D, T, B, varlen=True, max_seqlen=0, dtype=0):
+    a = native.SbaArgs()
+    a.dtype, a.head_dim, a.num_heads, a.num_seqs, a.total_tokens, a.max_seqlen = dtype, D, H, B, T, max_seqlen
+    a.cu_seqlens = 0x1000 if varlen else None        # only tested for NULL-ness by the size query
+    return a
+
+
+def test_workspace_sizes_cover_any_batch(native):
+    """The carry buffer is sized from (T, max_seqlen, num_seqs) alone; it must cover the exact need
+    sum_s 128 M_s (M_s + 1), M_s = ceil(L_s / 128), of every batch with those totals."""
+    lib = native.lib()
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        B = int(rng.integers(1, 40))
+        lengths = rng.integers(1, int(rng.choice([4, 70, 300, 5000])), size=B)
+        T, mx, H = int(lengths.sum()), int(lengths.max()), int(rng.integers(1, 9))
+        need = sum(128 * m * (m + 1) for m in (-(-int(n) // 128) for n in lengths)) * H * 4
+        fwd, bwd, carry = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+        for hint in (mx, 0):
+            a = _args(native, H, 64, T, B, max_seqlen=hint)
+            assert lib.sba_workspace_bytes(ctypes.byref(a), ctypes.byref(fwd), ctypes.byref(bwd), ctypes.byref(carry)) == 0
+            assert carry.value >= need and bwd.value >= fwd.value + carry.value
+            assert fwd.value >= 256 + 16 * (-(-T // 128) + B) + 8 * B
+    # fixed-length mode is exact
+    a = _args(native, 3, 128, 500, 4, varlen=False)
+    assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, ctypes.byref(carry)) == 0
+    assert carry.value == -(-(4 * 128 * 4 * 5 * 3 * 4) // 256) * 256
+
+
+def test_size_query_validates(native):
+    lib = native.lib()
+    assert lib.sba_workspace_bytes(None, None, None, None) == -1
+    assert lib.sba_workspace_bytes(ctypes.byref(_args(native, 0, 64, 10, 1)), None, None, None) == -6
+    assert lib.sba_workspace_bytes(ctypes.byref(_args(native, 1, 0, 10, 1)), None, None, None) == -3
+    assert lib.sba_workspace_bytes(ctypes.byref(_args(native, 1, 129, 10, 1)), None, None, None) == -3
+    assert lib.sba_workspace_bytes(ctypes.byref(_args(native, 1, 64, 10, 1, dtype=9)), None, None, None) == -2
+
+
+def test_operators_refuse_cpu_tensors(native):
+    from stickbreaking_attention import sb_attn, sb_attn_varlen
+
+    q = torch.zeros(2, 8, 16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        sb_attn_varlen(q, q, q, torch.tensor([8]), 8, zero_start=False)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        sb_attn(q[None], q[None], q[None])
+    with pytest.raises(AssertionError):
+        sb_attn_varlen(q, q, q, torch.tensor([3, 8]), 8, zero_start=True)
+
+
+def test_missing_library_fails_loudly(native, monkeypatch):
+    monkeypatch.setattr(native, "_lib", None)
+    monkeypatch.setattr(native, "_LIB_NAME", "libsba_absent.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        native.lib()
+
+
+def test_workload_generators():
+    import bench
+
+    for name, total, count in (("c1", 448, 3), ("c2", 16384, None), ("c3", 32768, None), ("c4", 32768, 8), ("c5", None, 2049)):
+        lengths = bench.lengths_for(name)
+        assert all(n >= 1 for n in lengths)
+        if total:
+            assert sum(lengths) == total
+        if count:
+            assert len(lengths) == count
+    assert max(bench.lengths_for("c3")) <= 8192 and bench.lengths_for("c5")[-1] == 16384
+    assert bench.visible_pairs([4096] * 8, 32) == 8 * 32 * 4096 * 4095 // 2 == 2146959360

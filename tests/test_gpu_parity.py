@@ -1,0 +1,308 @@
+"""GPU parity tests: the HIP path (through the C ABI, via the Python operators) against the CPU oracle on the
+same seeded inputs.
+
+Tolerances (stated here once): for 16-bit inputs the bar is max-abs error <= 2e-2 against the oracle evaluated
+in fp32/fp64 on the same bf16-rounded inputs.  A bf16 output cannot be closer to the true value than half a unit
+in the last place, which exceeds 2e-2 once |value| >= 4, so where |reference| is that large the bound is one bf16
+ulp of the reference (2^-7 |ref|) instead.  For fp32 inputs the bar is 1e-4.
+
+The adversarial configuration scales q and k by 3.  dq and dk are contractions of the 16-bit-rounded logit
+gradient against k and q (the reference rounds at the same point: sb_varlen_bwd.py:449-451), so their rounding
+noise grows with the operand magnitude; for those two tensors of that configuration the absolute part of the
+bound is scaled by the same factor 3 (6e-2), and the measured errors are printed.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import bench
+from oracle import sb_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ["o", "rem", "dq", "dk", "dv"]
+
+
+def tol_check(name, got, ref, dtype, label, operand_scale=1.0):
+    got = got.detach().double().cpu()
+    ref = ref.double()
+    assert not torch.isnan(got).any(), f"{label}: NaN in {name}"
+    err = (got - ref).abs()
+    if dtype == torch.float32:
+        bound = torch.full_like(ref, 1e-4)
+    elif dtype == torch.float16:
+        bound = torch.maximum(torch.full_like(ref, 2e-2), ref.abs() * 2.0 ** -10)
+    else:
+        absolute = 2e-2 * (operand_scale if name in ("dq", "dk") else 1.0)
+        bound = torch.maximum(torch.full_like(ref, absolute), ref.abs() * 2.0 ** -7)
+    worst = (err - bound).max().item()
+    print(f"{label} {name}: max-abs err {err.max().item():.3e} (ref max {ref.abs().max().item():.2f})", flush=True)
+    assert worst <= 0, f"{label}: {name} max-abs err {err.max().item():.4e} exceeds tolerance by {worst:.3e}"
+
+
+def run_varlen(q, k, v, cu, lengths, zero_start, attend_current, do, drem, scale=None, max_seqlens=True):
+    from stickbreaking_attention import sb_attn_varlen
+
+    q, k, v = (t.detach().clone().requires_grad_() for t in (q, k, v))
+    o, rem = sb_attn_varlen(q, k, v, cu, max(lengths) if max_seqlens else None, inv_temp=scale, zero_start=zero_start,
+                            attend_current=attend_current)
+    outs = [o, rem]
+    if do is not None:
+        outs += list(torch.autograd.grad([o, rem], [q, k, v], [do, drem]))
+    torch.cuda.synchronize()
+    return outs
+
+
+def small_case(H, D, lengths, dtype, seed, qk_std=1.0, device="cuda:0"):
+    g = torch.Generator().manual_seed(seed)
+    T = sum(lengths)
+    q, k, v, do = (torch.randn(H, T, D, generator=g) for _ in range(4))
+    drem = torch.randn(H, T, generator=g)
+    q, k = q * qk_std, k * qk_std
+    host = [t.to(dtype) for t in (q, k, v, do, drem)]
+    cu = torch.tensor(np.cumsum(lengths), dtype=torch.int32)
+    return host, [t.to(device) for t in host], cu
+
+
+SMALL = [
+    # label, H, D, lengths
+    ("single-key-tile", 1, 128, [64]),
+    ("one-query-tile", 2, 128, [128]),
+    ("ragged-with-length-1", 2, 128, [1, 5, 64, 65, 1, 128, 129, 300]),
+    ("d64", 3, 64, [200, 33, 500]),
+    ("odd-heads", 7, 128, [700, 100]),
+    ("d32", 2, 32, [257]),
+    ("d16", 2, 16, [130, 2]),
+    ("d50-unaligned", 2, 50, [100, 77]),
+    ("long-2k", 1, 128, [2048]),
+]
+
+
+@pytest.mark.parametrize("attend_current", [False, True])
+@pytest.mark.parametrize("label,H,D,lengths", SMALL)
+def test_small_bf16(gpu_device, label, H, D, lengths, attend_current):
+    host, dev, cu = small_case(H, D, lengths, torch.bfloat16, seed=1)
+    q, k, v, do, drem = host
+    ref = orc.varlen_stream(q, k, v, cu, attend_current=attend_current, do=do, drem=drem, dtype=torch.float64)
+    got = run_varlen(dev[0], dev[1], dev[2], cu.to(gpu_device), lengths, False, attend_current, dev[3], dev[4])
+    for n, a, b in zip(NAMES, got, ref):
+        tol_check(n, a, b, torch.bfloat16, label)
+
+
+def test_small_f16(gpu_device):
+    lengths = [300, 41]
+    host, dev, cu = small_case(2, 128, lengths, torch.float16, seed=2)
+    ref = orc.varlen_stream(*host[:3], cu, do=host[3], drem=host[4], dtype=torch.float64)
+    got = run_varlen(dev[0], dev[1], dev[2], cu.to(gpu_device), lengths, False, False, dev[3], dev[4])
+    for n, a, b in zip(NAMES, got, ref):
+        tol_check(n, a, b, torch.float16, "f16")
+
+
+def test_zero_start_forms_and_int64_cu_agree(gpu_device):
+    lengths = [77, 300, 1, 64]
+    host, dev, cu = small_case(4, 64, lengths, torch.bfloat16, seed=3)
+    cu = cu.to(gpu_device)
+    a = run_varlen(*dev[:3], cu, lengths, False, False, dev[3], dev[4])
+    cu0 = torch.cat([torch.zeros(1, dtype=torch.int64, device=gpu_device), cu.long()])
+    b = run_varlen(*dev[:3], cu0, lengths, True, False, dev[3], dev[4])
+    c = run_varlen(*dev[:3], cu, lengths, False, False, dev[3], dev[4], max_seqlens=False)     # README call form
+    for x, y, z in zip(a, b, c):
+        assert torch.equal(x, y) and torch.equal(x, z)
+    with pytest.raises(AssertionError):
+        run_varlen(*dev[:3], cu, lengths, True, False, None, None)      # cu[0] != 0, as the reference asserts
+
+
+def test_custom_scale_and_no_drem(gpu_device):
+    from stickbreaking_attention import sb_attn_varlen
+
+    lengths = [190, 66]
+    host, dev, cu = small_case(2, 128, lengths, torch.bfloat16, seed=4)
+    scale = 0.05
+    ref = orc.varlen_stream(*host[:3], cu, scale=scale, do=host[3], drem=torch.zeros_like(host[4]), dtype=torch.float64)
+    q, k, v = (t.clone().requires_grad_() for t in dev[:3])
+    o, rem = sb_attn_varlen(q, k, v, cu.to(gpu_device), max(lengths), inv_temp=scale, zero_start=False)
+    o.backward(dev[3])          # rem unused: autograd materialises a zero drem
+    for n, a, b in zip(NAMES, [o, rem, q.grad, k.grad, v.grad], ref):
+        tol_check(n, a, b, torch.bfloat16, "scale")
+
+
+def test_saturated_logits_long_row(gpu_device):
+    # q, k ~ N(0, 9): sigmoid saturates both ways; 3000 keys: the product of (1 - sigma) underflows early on most rows
+    lengths = [3000, 9]
+    host, dev, cu = small_case(2, 128, lengths, torch.bfloat16, seed=5, qk_std=3.0)
+    ref = orc.varlen_stream(*host[:3], cu, do=host[3], drem=host[4], dtype=torch.float64)
+    got = run_varlen(*dev[:3], cu.to(gpu_device), lengths, False, False, dev[3], dev[4])
+    for n, a, b in zip(NAMES, got, ref):
+        tol_check(n, a, b, torch.bfloat16, "saturated")
+
+
+def test_known_answers(gpu_device):
+    from stickbreaking_attention import sb_attn
+
+    # q = 0: A_ij = 2^-(i-j), rem_i = 2^-i (closed form); first row: o = 0, rem = 1
+    B, H, L, D = 1, 2, 200, 64
+    g = torch.Generator().manual_seed(6)
+    k = torch.randn(B, H, L, D, generator=g).bfloat16().to(gpu_device)
+    v = torch.randn(B, H, L, D, generator=g).bfloat16().to(gpu_device)
+    q = torch.zeros_like(k)
+    o, rem = sb_attn(q, k, v)
+    i = torch.arange(L, dtype=torch.float64)
+    torch.testing.assert_close(rem[0, 0].double().cpu(), 2.0 ** -i, atol=1e-3, rtol=2.0 ** -8)
+    w = torch.zeros(L, L, dtype=torch.float64)
+    for a in range(L):
+        for b in range(max(0, a - 60), a):
+            w[a, b] = 2.0 ** -(a - b)
+    expect = w @ v[0, 0].double().cpu()
+    assert (o[0, 0].double().cpu() - expect).abs().max() < 2e-2
+    assert (o[:, :, 0] == 0).all() and (rem[:, :, 0] == 1).all()
+    # strongly positive logits: all mass on the previous token
+    q = torch.ones_like(k) * 4
+    o, rem = sb_attn(q, torch.ones_like(k) * 4, v, inv_temp=1.0)
+    assert torch.equal(o[:, :, 1:], v[:, :, :-1]) and (rem[:, :, 1:].float() < 1e-29).all()
+
+
+@pytest.mark.parametrize("attend_current", [False, True])
+def test_fixed_length_matches_oracle_and_varlen(gpu_device, attend_current):
+    from stickbreaking_attention import sb_attn
+
+    B, H, L, D = 3, 2, 500, 64          # 500: partial tiles, as tests/test_attn.py:45 exercises
+    g = torch.Generator().manual_seed(7)
+    q, k, v, do = (torch.randn(B, H, L, D, generator=g).bfloat16() for _ in range(4))
+    drem = torch.randn(B, H, L, generator=g).bfloat16()
+    ref = orc.fixed_stream(q, k, v, attend_current=attend_current, do=do, drem=drem, dtype=torch.float64)
+    qd, kd, vd = (t.to(gpu_device).requires_grad_() for t in (q, k, v))
+    o, rem = sb_attn(qd, kd, vd, attend_current=attend_current)
+    grads = torch.autograd.grad([o, rem], [qd, kd, vd], [do.to(gpu_device), drem.to(gpu_device)])
+    for n, a, b in zip(NAMES, [o, rem, *grads], ref):
+        tol_check(n, a, b, torch.bfloat16, "fixed")
+    # the same data packed as B sequences of one varlen batch gives bit-identical results
+    pack = lambda t: t.transpose(0, 1).reshape(H, B * L, -1)
+    cu = torch.arange(1, B + 1, dtype=torch.int32, device=gpu_device) * L
+    got = run_varlen(pack(qd), pack(kd), pack(vd), cu, [L] * B, False, attend_current, pack(do.to(gpu_device)),
+                     drem.to(gpu_device).transpose(0, 1).reshape(H, B * L))
+    assert torch.equal(got[0], pack(o)) and torch.equal(got[2], pack(grads[0])) and torch.equal(got[3], pack(grads[1]))
+
+
+def test_strided_token_major_inputs(gpu_device):
+    # benchmarks/varlen.py:44-46 hands (T, H, D) tensors permuted to (H, T, D): non-contiguous head/token strides
+    lengths = [150, 90]
+    host, dev, cu = small_case(4, 64, lengths, torch.bfloat16, seed=8)
+    a = run_varlen(*dev[:3], cu.to(gpu_device), lengths, False, False, dev[3], dev[4])
+    thd = [t.transpose(0, 1).contiguous().transpose(0, 1) for t in dev[:4]]
+    b = run_varlen(*thd[:3], cu.to(gpu_device), lengths, False, False, thd[3], dev[4])
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    assert b[0].stride() == thd[0].stride()        # o keeps q's layout (empty_like, sb_varlen_fwd.py:417)
+
+
+def _full_size(name, gpu_device, oracle_heads, bwd=True, attend_current=False):
+    inp = bench.make_inputs(name, gpu_device)
+    lengths, H = inp["lengths"], inp["H"]
+    got = run_varlen(inp["q"], inp["k"], inp["v"], inp["cu"], lengths, inp["zero_start"], attend_current,
+                     inp["do"] if bwd else None, inp["drem"] if bwd else None)
+    for t in got:
+        assert torch.isfinite(t.float()).all()
+    rem = got[1].float()
+    assert (rem >= 0).all() and (rem <= 1).all()
+    starts = np.concatenate([[0], np.cumsum(lengths)[:-1]])
+    st = torch.tensor(starts, device=gpu_device)
+    assert (got[0][:, st] == 0).all() and (rem[:, st] == 1).all()        # first token of every sequence
+    cu_host = inp["cu"].cpu()
+    host = [inp[n].cpu() for n in ("q", "k", "v", "do", "drem")]
+    ref = orc.varlen_stream(host[0], host[1], host[2], cu_host, zero_start=inp["zero_start"], attend_current=attend_current,
+                            do=host[3] if bwd else None, drem=host[4] if bwd else None, dtype=torch.float32, heads=oracle_heads)
+    for n, a, b in zip(NAMES, got, ref):
+        tol_check(n, a[oracle_heads], b[oracle_heads], inp["dtype"], f"{name} heads {oracle_heads}")
+    return inp, got
+
+
+def test_config2_forward_full_size(gpu_device):
+    _full_size("c2", gpu_device, [0, 5, 11], bwd=False)
+
+
+def test_config3_full_size(gpu_device):
+    inp, got = _full_size("c3", gpu_device, [0, 17, 31])
+    # size-independent property over ALL heads: each sequence on its own (fixed-length entry point) reproduces
+    # its slice of the packed result bit for bit
+    from stickbreaking_attention import sb_attn
+
+    longest = int(np.argmax(inp["lengths"]))
+    s0 = int(np.sum(inp["lengths"][:longest]))
+    n = inp["lengths"][longest]
+    q, k, v = (inp[x][:, s0:s0 + n].unsqueeze(0) for x in ("q", "k", "v"))
+    o, rem = sb_attn(q, k, v)
+    assert torch.equal(o[0], got[0][:, s0:s0 + n]) and torch.equal(rem[0], got[1][:, s0:s0 + n])
+
+
+def test_config4_fixed_full_size(gpu_device):
+    from stickbreaking_attention import sb_attn
+
+    inp = bench.make_inputs("c4", gpu_device)
+    H, D, B, L = inp["H"], inp["D"], 8, 4096
+    view = lambda t: t.view(H, B, L, -1).transpose(0, 1)
+    q, k, v = (view(inp[n]).requires_grad_() for n in ("q", "k", "v"))
+    o, rem = sb_attn(q, k, v)
+    do, drem = view(inp["do"]), inp["drem"].view(H, B, L).transpose(0, 1)
+    grads = torch.autograd.grad([o, rem], [q, k, v], [do, drem])
+    for t in (o, rem, *grads):
+        assert torch.isfinite(t.float()).all()
+    # oracle on two (batch, head) slices
+    for b, h in ((0, 0), (7, 31)):
+        sl = [t[b:b + 1, h:h + 1].detach().cpu() for t in (q, k, v, do)]
+        ref = orc.fixed_stream(*sl[:3], do=sl[3], drem=drem[b:b + 1, h:h + 1].cpu(), dtype=torch.float32)
+        got = [o, rem, *grads]
+        for n, a, r in zip(NAMES, got, ref):
+            tol_check(n, a[b:b + 1, h:h + 1], r, torch.bfloat16, f"c4[{b},{h}]")
+
+
+def test_config5_adversarial_ragged(gpu_device):
+    # 2048 sequences of 1..64 tokens plus one of 16384, zero_start=True, saturating logits.
+    # The oracle covers every short sequence on two heads and the long sequence on one head.
+    inp = bench.make_inputs("c5", gpu_device)
+    lengths = inp["lengths"]
+    got = run_varlen(inp["q"], inp["k"], inp["v"], inp["cu"], lengths, True, False, inp["do"], inp["drem"])
+    for t in got:
+        assert torch.isfinite(t.float()).all()
+    short_T = sum(lengths[:-1])
+    host = [inp[n].cpu() for n in ("q", "k", "v", "do", "drem")]
+    cu_short = torch.tensor(np.cumsum(lengths[:-1]))
+    heads = [3, 30]
+    ref = orc.varlen_stream(*(t[:, :short_T] for t in host[:3]), cu_short, do=host[3][:, :short_T], drem=host[4][:, :short_T],
+                            dtype=torch.float32, heads=heads)
+    for n, a, b in zip(NAMES, got, ref):
+        tol_check(n, a[heads, :short_T], b[heads], torch.bfloat16, "c5 short sequences", operand_scale=3.0)
+    h = 9
+    sl = [t[h:h + 1, short_T:] for t in host]
+    ref = orc.varlen_stream(sl[0], sl[1], sl[2], [lengths[-1]], do=sl[3], drem=sl[4], dtype=torch.float32)
+    for n, a, b in zip(NAMES, got, ref):
+        tol_check(n, a[h:h + 1, short_T:], b, torch.bfloat16, "c5 long sequence", operand_scale=3.0)
+
+
+def test_forward_without_grad_skips_carry(gpu_device):
+    from stickbreaking_attention import _native
+
+    host, dev, cu = small_case(2, 64, [100], torch.bfloat16, seed=9)
+    o, rem, stat, carry = _native.forward(dev[0], dev[1], dev[2], cu.to(gpu_device), False, 100, 0.125, False, want_carry=False)
+    assert carry is None
+    torch.testing.assert_close(torch.exp2(stat), rem.float(), atol=4e-3, rtol=4e-3)   # row_stat = log2(rem)
+
+
+def test_c_abi_rejects_bad_arguments(gpu_device):
+    import ctypes
+
+    from stickbreaking_attention import _native
+
+    lib = _native.lib()
+    a = _native.SbaArgs()
+    a.dtype, a.head_dim, a.num_heads, a.num_seqs, a.total_tokens = 0, 256, 2, 1, 64
+    assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, None) == -3          # head_dim
+    a.head_dim, a.dtype = 64, 7
+    assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, None) == -2          # dtype
+    a.dtype = 0
+    assert lib.sba_fwd(ctypes.byref(a)) == -1                                        # NULL tensors
+    assert lib.sba_fwd(None) == -1
+    q = torch.zeros(2, 64, 64, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(RuntimeError):
+        _native.forward(q.cpu(), q.cpu(), q.cpu(), None, False, 0, 1.0, False, False)
