@@ -17,8 +17,8 @@
 namespace sba {
 
 template <int DH> struct DkvLds {
-  static constexpr int kRowStride = DH + kPad;
-  static constexpr int kPStride = kBlockK + kPad;
+  static constexpr int kRowStride = lds_stride<DH>();
+  static constexpr int kPStride = lds_stride<kBlockK>();
   static constexpr int kQ = 0;
   static constexpr int kDo = kQ + kBlockQ * kRowStride;
   static constexpr int kK = kDo + kBlockQ * kRowStride;
@@ -28,7 +28,7 @@ template <int DH> struct DkvLds {
   static constexpr int kElems = kDz + kBlockQ * kPStride;
 };
 
-template <typename T, int DH>
+template <typename T, int DH, bool kFast>
 __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
   typedef typename Elem<T>::vec8 vec8;
   typedef DkvLds<DH> Lds;
@@ -50,7 +50,6 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
   const Tile tile = p.k_tiles[slot];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, col = lane & 31;
   const int L = tile.seq_len, j0 = tile.origin, ac = p.attend_current, D = p.head_dim;
-  const bool vec_ok = p.vec_ok != 0;
   const int64_t tok0 = tile.seq_start;
   const int jt = j0 / kBlockK;
 
@@ -70,9 +69,9 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
     for (int r = 0; r < 16; r++) { dkacc[b][r] = 0.f; dvacc[b][r] = 0.f; }
 
   {
-    TileCopy<T, DH, kBlockK> ck, cv;
-    ck.load(kb + (int64_t)j0 * p.k.st, p.k.st, L - j0, D, vec_ok);
-    cv.load(vb + (int64_t)j0 * p.v.st, p.v.st, L - j0, D, vec_ok);
+    TileCopy<T, DH, kBlockK, kFast> ck, cv;
+    ck.load(kb + (int64_t)j0 * p.k.st, p.k.st, L - j0, D);
+    cv.load(vb + (int64_t)j0 * p.v.st, p.v.st, L - j0, D);
     ck.store(k_lds);
     cv.store(v_lds);
   }
@@ -89,10 +88,10 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
     const int q0 = qt * kBlockQ;
     __syncthreads();      // previous contraction finished reading q/do/p/dz tiles
     {
-      TileCopy<T, DH, kBlockQ> cq;
-      cq.load(qb + (int64_t)q0 * p.q.st, p.q.st, L - q0, D, vec_ok);
+      TileCopy<T, DH, kBlockQ, kFast> cq;
+      cq.load(qb + (int64_t)q0 * p.q.st, p.q.st, L - q0, D);
       cq.store(q_lds);
-      cq.load(dob + (int64_t)q0 * p.d_o.st, p.d_o.st, L - q0, D, vec_ok);
+      cq.load(dob + (int64_t)q0 * p.d_o.st, p.d_o.st, L - q0, D);
       cq.store(do_lds);
     }
     __syncthreads();
@@ -179,21 +178,23 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
   }
 }
 
-template <typename T, int DH>
+template <typename T, int DH, bool kFast>
 static hipError_t launch_one(const BwdParams& p, int max_tiles, hipStream_t stream) {
   const size_t lds_bytes = (size_t)DkvLds<DH>::kElems * sizeof(T);
   // The tile set exceeds the default 64 KB dynamic-LDS cap; the attribute is per device and cheap to set.
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv_kernel<T, DH>),
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv_kernel<T, DH, kFast>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (e != hipSuccess) return e;
   const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kThreads);
-  hipLaunchKernelGGL((bwd_dkv_kernel<T, DH>), grid, block, lds_bytes, stream, p);
+  hipLaunchKernelGGL((bwd_dkv_kernel<T, DH, kFast>), grid, block, lds_bytes, stream, p);
   return hipGetLastError();
 }
 
 template <typename T>
 static hipError_t launch_t(const BwdParams& p, int max_tiles, hipStream_t stream) {
-  return p.head_dim <= 64 ? launch_one<T, 64>(p, max_tiles, stream) : launch_one<T, 128>(p, max_tiles, stream);
+  if (p.vec_ok && p.head_dim == 128) return launch_one<T, 128, true>(p, max_tiles, stream);
+  if (p.vec_ok && p.head_dim == 64) return launch_one<T, 64, true>(p, max_tiles, stream);
+  return p.head_dim <= 64 ? launch_one<T, 64, false>(p, max_tiles, stream) : launch_one<T, 128, false>(p, max_tiles, stream);
 }
 
 hipError_t launch_bwd_dkv(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream) {

@@ -19,10 +19,10 @@
 
 namespace sba {
 
-template <typename T, int DH>
+template <typename T, int DH, bool kFast>
 __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
   typedef typename Elem<T>::vec8 vec8;
-  constexpr int kRowStride = DH + kPad;
+  constexpr int kRowStride = lds_stride<DH>();
   constexpr int kSteps = DH / 16;
   constexpr int kDTiles = DH / 32;
   __shared__ __attribute__((aligned(16))) T k_lds[kBlockK * kRowStride];
@@ -34,7 +34,6 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
   const Tile tile = p.q_tiles[slot];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, col = lane & 31;
   const int L = tile.seq_len, q0 = tile.origin, ac = p.attend_current, D = p.head_dim;
-  const bool vec_ok = p.vec_ok != 0;
   const int64_t tok0 = tile.seq_start;
 
   const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
@@ -48,8 +47,8 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
 #pragma unroll
   for (int kk = 0; kk < kSteps; kk++) {
     const int d0 = 16 * kk + 8 * half;
-    qf[kk] = as_vec8<T>(load_row8<T>(qb + (int64_t)qi * p.q.st, d0, D, row_ok, vec_ok));
-    dof[kk] = as_vec8<T>(load_row8<T>(dob + (int64_t)qi * p.d_o.st, d0, D, row_ok, vec_ok));
+    qf[kk] = as_vec8<T>(load_row8<T, kFast>(qb + (int64_t)qi * p.q.st, d0, D, row_ok));
+    dof[kk] = as_vec8<T>(load_row8<T, kFast>(dob + (int64_t)qi * p.d_o.st, d0, D, row_ok));
   }
   float drem = 0.f;
   if (row_ok && p.d_rem.ptr)
@@ -71,10 +70,10 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
 #pragma unroll
     for (int r = 0; r < 16; r++) dqacc[dt][r] = 0.f;
 
-  TileCopy<T, DH, kBlockK> ck, cv;
+  TileCopy<T, DH, kBlockK, kFast> ck, cv;
   if (n_kt > 0) {
-    ck.load(kb, p.k.st, L, D, vec_ok);
-    cv.load(vb, p.v.st, L, D, vec_ok);
+    ck.load(kb, p.k.st, L, D);
+    cv.load(vb, p.v.st, L, D);
   }
   for (int jt = 0; jt < n_kt; ++jt) {
     const int j0 = jt * kBlockK;
@@ -84,8 +83,8 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
     __syncthreads();
     if (jt + 1 < n_kt) {
       const int jn = j0 + kBlockK;
-      ck.load(kb + (int64_t)jn * p.k.st, p.k.st, L - jn, D, vec_ok);
-      cv.load(vb + (int64_t)jn * p.v.st, p.v.st, L - jn, D, vec_ok);
+      ck.load(kb + (int64_t)jn * p.k.st, p.k.st, L - jn, D);
+      cv.load(vb + (int64_t)jn * p.v.st, p.v.st, L - jn, D);
     }
     // For the key-stationary kernel: C just below this tile, for every row of the tile.
     const int64_t slot_idx = carry_offset(jt, n_qt) + (qi - kBlockQ * (jt >> 1));
@@ -142,10 +141,14 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
 template <typename T>
 static hipError_t launch_t(const BwdParams& p, int max_tiles, hipStream_t stream) {
   const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kThreads);
-  if (p.head_dim <= 64) {
-    hipLaunchKernelGGL((bwd_dq_kernel<T, 64>), grid, block, 0, stream, p);
+  if (p.vec_ok && p.head_dim == 128) {
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 128, true>), grid, block, 0, stream, p);
+  } else if (p.vec_ok && p.head_dim == 64) {
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 64, true>), grid, block, 0, stream, p);
+  } else if (p.head_dim <= 64) {
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 64, false>), grid, block, 0, stream, p);
   } else {
-    hipLaunchKernelGGL((bwd_dq_kernel<T, 128>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 128, false>), grid, block, 0, stream, p);
   }
   return hipGetLastError();
 }

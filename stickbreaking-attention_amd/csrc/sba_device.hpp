@@ -84,8 +84,11 @@ __device__ __forceinline__ float other_half(float x, int half) {
   return __builtin_bit_cast(float, o);
 }
 
-// LDS row-major tile of 16-bit elements with `kPad` elements of padding per row.
-constexpr int kPad = 8;
+// LDS row-major tiles of 16-bit elements.  Row strides of 304 bytes (128 + 24 elements) and 144 bytes
+// (64 + 8 elements) were measured conflict-free for both access patterns used here: 16-byte reads along 16
+// consecutive rows (MFMA operands contracted over the row) and the 8-byte transpose reads that gather an
+// operand down 4 consecutive rows.  (272 bytes halves the transpose-read rate; 288 and 320 hurt the row reads.)
+template <int W> constexpr int lds_stride() { return W == 128 ? 152 : W + 8; }
 
 // 8 consecutive elements of one row (A operand for contractions over head_dim, or over a row's own axis).
 template <typename T>
@@ -118,8 +121,9 @@ __device__ __forceinline__ int mfma_row_to_key(int mt, int m) {
 }
 
 // Cooperative global -> register -> LDS copy of a [kRows x DH] tile of 16-bit elements, 16 bytes per access.
-// Rows at or beyond `rows_valid` and columns at or beyond `d_valid` are zero-filled.
-template <typename T, int DH, int kRows>
+// kFast: head_dim == DH and every row start is 16-byte aligned, so the copy is straight-line 16-byte loads.
+// Otherwise rows at or beyond `rows_valid` (>= 1) and columns at or beyond `d_valid` are zero-filled.
+template <typename T, int DH, int kRows, bool kFast>
 struct TileCopy {
   static constexpr int kChunksPerRow = DH / 8;
   static constexpr int kChunks = kRows * kChunksPerRow;
@@ -127,25 +131,28 @@ struct TileCopy {
   static_assert(kChunks % kThreads == 0, "tile must divide evenly over the workgroup");
   u32x4 regs[kPerThread];
 
-  __device__ __forceinline__ void load(const T* base, int64_t row_stride, int rows_valid, int d_valid, bool vec_ok) {
+  __device__ __forceinline__ void load(const T* base, int64_t row_stride, int rows_valid, int d_valid) {
 #pragma unroll
     for (int i = 0; i < kPerThread; i++) {
       const int c = threadIdx.x + i * kThreads;
       const int row = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
-      u32x4 v = {0, 0, 0, 0};
-      if (row < rows_valid) {
-        const T* p = base + row * row_stride + col;
-        if (vec_ok && col + 8 <= d_valid) {
-          v = *reinterpret_cast<const u32x4*>(p);
-        } else {
+      if (kFast) {
+        // Out-of-range rows re-read the last valid row: finite data that every consumer masks (a key beyond the
+        // sequence is hidden from every row; a query row beyond it is forced hidden) -- no zero fill needed.
+        const int rr = min(row, rows_valid - 1);
+        regs[i] = *reinterpret_cast<const u32x4*>(base + rr * row_stride + col);
+      } else {
+        u32x4 v = {0, 0, 0, 0};
+        if (row < rows_valid) {
+          const uint16_t* p = reinterpret_cast<const uint16_t*>(base + row * row_stride + col);
           uint16_t e[8];
 #pragma unroll
-          for (int t = 0; t < 8; t++) e[t] = (col + t < d_valid) ? reinterpret_cast<const uint16_t*>(p)[t] : (uint16_t)0;
+          for (int t = 0; t < 8; t++) e[t] = (col + t < d_valid) ? p[t] : (uint16_t)0;
           v[0] = e[0] | ((uint32_t)e[1] << 16); v[1] = e[2] | ((uint32_t)e[3] << 16);
           v[2] = e[4] | ((uint32_t)e[5] << 16); v[3] = e[6] | ((uint32_t)e[7] << 16);
         }
+        regs[i] = v;
       }
-      regs[i] = v;
     }
   }
   __device__ __forceinline__ void store(T* tile) const {
@@ -153,17 +160,17 @@ struct TileCopy {
     for (int i = 0; i < kPerThread; i++) {
       const int c = threadIdx.x + i * kThreads;
       const int row = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
-      *reinterpret_cast<u32x4*>(tile + row * (DH + kPad) + col) = regs[i];
+      *reinterpret_cast<u32x4*>(tile + row * lds_stride<DH>() + col) = regs[i];
     }
   }
 };
 
 // Load 8 consecutive head_dim elements of one token row from global memory (zero beyond head_dim / when !valid).
-template <typename T>
-__device__ __forceinline__ u32x4 load_row8(const T* row, int d0, int d_valid, bool valid, bool vec_ok) {
+template <typename T, bool kFast>
+__device__ __forceinline__ u32x4 load_row8(const T* row, int d0, int d_valid, bool valid) {
   u32x4 v = {0, 0, 0, 0};
   if (valid) {
-    if (vec_ok && d0 + 8 <= d_valid) {
+    if (kFast) {
       v = *reinterpret_cast<const u32x4*>(row + d0);
     } else {
       uint16_t e[8];
@@ -187,45 +194,56 @@ constexpr float kExpClamp = 100.0f;   // 2^100 and 2^-100 are finite; sigma(z) i
 // Produces P (pk) and dZ = g - sigma * C (dzk), C_ij = sum_{j' <= j} g_ij', packed to 16 bit two keys per
 // word, and the prefix sum for the next tile up.  (The reference evaluates the same quantities tile by tile at
 // stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:438-447.)
-template <typename T>
-__device__ __forceinline__ void bwd_tile_math(const f32x16 (&s)[2], const f32x16 (&dp)[2], float scale_log2, bool diagonal,
-                                              int lim, int half, float drem, float prod_in, float prefix_in,
-                                              uint32_t (&pk)[16], uint32_t (&dzk)[16], float& prefix_out) {
-  float beta[32], pr[32], cum[32];
+template <typename T, bool kDiagonal>
+__device__ __forceinline__ void bwd_tile_math_impl(const f32x16 (&s)[2], const f32x16 (&dp)[2], float scale_log2, int lim,
+                                                   int half, float drem, float prod_in, float prefix_in,
+                                                   uint32_t (&pk)[16], uint32_t (&dzk)[16], float& prefix_out) {
+  // sigma = 1 - 1/(1+e) needs no clamp on e: e = inf gives 1/(1+e) = 0 and sigma = 1 exactly, and the absolute
+  // error of the subtraction (6e-8) is far below the 16-bit rounding of P and dZ.
+  float beta[32], pe[32];
   float run = 1.f;
 #pragma unroll
   for (int R = 31; R >= 0; --R) {
     float x = s[R >> 4][R & 15] * scale_log2;
-    x = fast_min(x, kExpClamp);
-    if (diagonal) x = (R < lim) ? x : -INFINITY;
-    const float e = fast_exp2(x);
-    const float omb = fast_rcp(1.f + e);
-    beta[R] = e * omb;
-    pr[R] = run;           // product over this lane's higher keys
+    if (kDiagonal) x = (R < lim) ? x : -INFINITY;
+    const float omb = fast_rcp(1.f + fast_exp2(x));
+    beta[R] = 1.f - omb;
+    pe[R] = run;           // product over this lane's higher keys
     run *= omb;
   }
   const float oth = other_half(run, half);
   const float seed = half ? prod_in : prod_in * oth;      // the upper half-wave holds the higher keys
-  float acc = 0.f;
+  // Running C as if this lane's keys were preceded only by the keys below the tile; the upper half-wave's
+  // share of the lower half-wave's total is added afterwards (fixup).
+  float acc = prefix_in;
+  float dz[32];
 #pragma unroll
   for (int R = 0; R < 32; R++) {
-    const float a = beta[R] * (pr[R] * seed);
-    pr[R] = a;
-    acc += a * (dp[R >> 4][R & 15] - drem);
-    cum[R] = acc;          // inclusive prefix sum of g over this lane's keys
+    const float a = beta[R] * (pe[R] * seed);
+    const float g = a * (dp[R >> 4][R & 15] - drem);
+    acc += g;
+    dz[R] = g - beta[R] * acc;
+    pe[R] = a;
   }
-  const float oth_g = other_half(acc, half);
-  const float base = half ? prefix_in + oth_g : prefix_in;  // the lower half-wave holds the lower keys
-  prefix_out = prefix_in + (acc + oth_g);
+  const float tot = acc - prefix_in;
+  const float oth_g = other_half(tot, half);
+  const float fixup = half ? oth_g : 0.f;                   // the lower half-wave holds the lower keys
+  prefix_out = acc + oth_g;
 #pragma unroll
   for (int R = 0; R < 32; R += 2) {
-    const float g0 = cum[R] - (R ? cum[R - 1] : 0.f);
-    const float g1 = cum[R + 1] - cum[R];
-    const float dz0 = g0 - beta[R] * (base + cum[R]);
-    const float dz1 = g1 - beta[R + 1] * (base + cum[R + 1]);
-    pk[R >> 1] = pack2<T>(pr[R], pr[R + 1]);
-    dzk[R >> 1] = pack2<T>(dz0, dz1);
+    pk[R >> 1] = pack2<T>(pe[R], pe[R + 1]);
+    dzk[R >> 1] = pack2<T>(dz[R] - beta[R] * fixup, dz[R + 1] - beta[R + 1] * fixup);
   }
+}
+
+template <typename T>
+__device__ __forceinline__ void bwd_tile_math(const f32x16 (&s)[2], const f32x16 (&dp)[2], float scale_log2, bool diagonal,
+                                              int lim, int half, float drem, float prod_in, float prefix_in,
+                                              uint32_t (&pk)[16], uint32_t (&dzk)[16], float& prefix_out) {
+  if (diagonal)
+    bwd_tile_math_impl<T, true>(s, dp, scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prefix_out);
+  else
+    bwd_tile_math_impl<T, false>(s, dp, scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prefix_out);
 }
 
 // Map the linear workgroup id to (head, tile slot) so that the workgroups of one head land on one XCD

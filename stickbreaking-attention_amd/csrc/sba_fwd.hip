@@ -16,10 +16,10 @@
 
 namespace sba {
 
-template <typename T, int DH>
-__global__ __launch_bounds__(kThreads) void fwd_kernel(FwdParams p) {
+template <typename T, int DH, bool kFast>
+__global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FwdParams p) {
   typedef typename Elem<T>::vec8 vec8;
-  constexpr int kRowStride = DH + kPad;
+  constexpr int kRowStride = lds_stride<DH>();
   constexpr int kSteps = DH / 16;    // MFMA k-steps over head_dim
   constexpr int kDTiles = DH / 32;   // 32-wide output tiles over head_dim
   __shared__ __attribute__((aligned(16))) T k_lds[kBlockK * kRowStride];
@@ -31,7 +31,6 @@ __global__ __launch_bounds__(kThreads) void fwd_kernel(FwdParams p) {
   const Tile tile = p.tiles[slot];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, col = lane & 31;
   const int L = tile.seq_len, q0 = tile.origin, ac = p.attend_current, D = p.head_dim;
-  const bool vec_ok = p.vec_ok != 0;
 
   const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + (int64_t)tile.seq_start * p.q.st;
   const T* kb = (const T*)p.k.ptr + tile.seq_id * p.k.sb + head * p.k.sh + (int64_t)tile.seq_start * p.k.st;
@@ -42,7 +41,7 @@ __global__ __launch_bounds__(kThreads) void fwd_kernel(FwdParams p) {
   vec8 qf[kSteps];
 #pragma unroll
   for (int kk = 0; kk < kSteps; kk++)
-    qf[kk] = as_vec8<T>(load_row8<T>(qb + (int64_t)qi * p.q.st, 16 * kk + 8 * half, D, qi < L, vec_ok));
+    qf[kk] = as_vec8<T>(load_row8<T, kFast>(qb + (int64_t)qi * p.q.st, 16 * kk + 8 * half, D, qi < L));
 
   const int last_row = min(q0 + kBlockQ, L) - 1;
   const int last_key = last_row - 1 + ac;                    // last key any row of this tile can see
@@ -58,11 +57,11 @@ __global__ __launch_bounds__(kThreads) void fwd_kernel(FwdParams p) {
   const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
   float* carry = p.carry ? p.carry + (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] : nullptr;
 
-  TileCopy<T, DH, kBlockK> ck, cv;
+  TileCopy<T, DH, kBlockK, kFast> ck, cv;
   if (n_kt > 0) {
     const int j0 = (n_kt - 1) * kBlockK;
-    ck.load(kb + (int64_t)j0 * p.k.st, p.k.st, L - j0, D, vec_ok);
-    cv.load(vb + (int64_t)j0 * p.v.st, p.v.st, L - j0, D, vec_ok);
+    ck.load(kb + (int64_t)j0 * p.k.st, p.k.st, L - j0, D);
+    cv.load(vb + (int64_t)j0 * p.v.st, p.v.st, L - j0, D);
   }
   for (int jt = n_kt - 1; jt >= 0; --jt) {
     const int j0 = jt * kBlockK;
@@ -72,8 +71,8 @@ __global__ __launch_bounds__(kThreads) void fwd_kernel(FwdParams p) {
     __syncthreads();
     if (jt > 0) {
       const int jn = j0 - kBlockK;
-      ck.load(kb + (int64_t)jn * p.k.st, p.k.st, L - jn, D, vec_ok);
-      cv.load(vb + (int64_t)jn * p.v.st, p.v.st, L - jn, D, vec_ok);
+      ck.load(kb + (int64_t)jn * p.k.st, p.k.st, L - jn, D);
+      cv.load(vb + (int64_t)jn * p.v.st, p.v.st, L - jn, D);
     }
     // For the backward: the product over the keys between this tile and the row, for every row of the tile.
     if (carry && half == 0) carry[carry_offset(jt, n_qt) + (qi - kBlockQ * (jt >> 1))] = prod;
@@ -94,38 +93,40 @@ __global__ __launch_bounds__(kThreads) void fwd_kernel(FwdParams p) {
       }
     }
 
-    // e = 2^x for this lane's 32 keys j0 + 32*half + R, R = 16*mt + r; hidden keys get e = 0 (factor 1, weight 0).
-    float e[32];
-    const int lim = qi + ac - j0 - 32 * half;                 // key R is visible iff R < lim
-#pragma unroll
-    for (int R = 0; R < 32; R++) {
-      float x = s[R >> 4][R & 15] * p.scale_log2;
-      x = fast_min(x, kExpClamp);
-      if (diagonal) x = (R < lim) ? x : -INFINITY;
-      e[R] = fast_exp2(x);
-    }
-    // w[R] = prod_{R' >= R} 1/(1+e[R'])  (reverse inclusive scan along this lane's keys)
-    float w[32];
+    // This lane's 32 keys are j0 + 32*half + R, R = 16*mt + r, swept from R = 31 down.
+    //   t[R] = e[R] * prod_{R' >= R} 1/(1+e[R'])   (the weight of key R up to the product carried into the tile)
+    // Hidden keys (diagonal tiles only) get e = 0: factor 1, weight 0.
+    float t[32];
     float run = 1.f;
+    if (diagonal) {
+      const int lim = qi + ac - j0 - 32 * half;               // key R is visible iff R < lim
 #pragma unroll
-    for (int R = 31; R >= 0; --R) {
-      const float omb = fast_rcp(1.f + e[R]);
-      run = (R == 31) ? omb : run * omb;
-      w[R] = run;
+      for (int R = 31; R >= 0; --R) {
+        float x = fast_min(s[R >> 4][R & 15] * p.scale_log2, kExpClamp);
+        x = (R < lim) ? x : -INFINITY;
+        const float e = fast_exp2(x);
+        run *= fast_rcp(1.f + e);
+        t[R] = e * run;
+      }
+    } else {
+#pragma unroll
+      for (int R = 31; R >= 0; --R) {
+        const float e = fast_exp2(fast_min(s[R >> 4][R & 15] * p.scale_log2, kExpClamp));
+        run *= fast_rcp(1.f + e);
+        t[R] = e * run;
+      }
     }
     const float oth = other_half(run, half);
     // The upper half-wave holds the higher keys, which come first in the sweep.
     const float seed = half ? prod : prod * oth;
     prod = (prod * oth) * run;
 
-    uint32_t pk[16];
-#pragma unroll
-    for (int R = 0; R < 32; R += 2) pk[R >> 1] = pack2<T>(e[R] * (w[R] * seed), e[R + 1] * (w[R + 1] * seed));
-
     // O += P V: A = P from registers (k index <-> key 32*half + 8c + t), B = V gathered down the keys.
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-      u32x4 av = {pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
+      u32x4 av;
+#pragma unroll
+      for (int i = 0; i < 4; i++) av[i] = pack2<T>(t[8 * c + 2 * i] * seed, t[8 * c + 2 * i + 1] * seed);
       vec8 a = as_vec8<T>(av);
 #pragma unroll
       for (int dt = 0; dt < kDTiles; dt++) {
@@ -154,19 +155,23 @@ __global__ __launch_bounds__(kThreads) void fwd_kernel(FwdParams p) {
 }
 
 template <typename T>
-static hipError_t launch_fwd_t(const FwdParams& p, int dh, int max_tiles, hipStream_t stream) {
+static hipError_t launch_fwd_t(const FwdParams& p, int max_tiles, hipStream_t stream) {
   const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kThreads);
-  if (dh <= 64) {
-    hipLaunchKernelGGL((fwd_kernel<T, 64>), grid, block, 0, stream, p);
+  if (p.vec_ok && p.head_dim == 128) {
+    hipLaunchKernelGGL((fwd_kernel<T, 128, true>), grid, block, 0, stream, p);
+  } else if (p.vec_ok && p.head_dim == 64) {
+    hipLaunchKernelGGL((fwd_kernel<T, 64, true>), grid, block, 0, stream, p);
+  } else if (p.head_dim <= 64) {
+    hipLaunchKernelGGL((fwd_kernel<T, 64, false>), grid, block, 0, stream, p);
   } else {
-    hipLaunchKernelGGL((fwd_kernel<T, 128>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<T, 128, false>), grid, block, 0, stream, p);
   }
   return hipGetLastError();
 }
 
 hipError_t launch_fwd(const FwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream) {
-  return dtype_is_f16 ? launch_fwd_t<_Float16>(p, p.head_dim, max_tiles, stream)
-                      : launch_fwd_t<__bf16>(p, p.head_dim, max_tiles, stream);
+  return dtype_is_f16 ? launch_fwd_t<_Float16>(p, max_tiles, stream)
+                      : launch_fwd_t<__bf16>(p, max_tiles, stream);
 }
 
 }  // namespace sba
