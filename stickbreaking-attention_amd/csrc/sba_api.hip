@@ -43,8 +43,8 @@ int plan(const SbaArgs* a, Layout* out) {
   } else {
     L.max_q_tiles = cdiv(T, kBlockQ) + B;
     L.max_k_tiles = cdiv(T, kBlockK) + B;
-    // sum_s 128 M_s (M_s + 1) with M_s <= L_s/128 + 1 and sum_s L_s^2 <= T * max_len
-    L.carry_slots_per_head = cdiv(T * max_len, 128) + 3 * T + 256 * B;
+    // sum_s 256 M_s (M_s + 1) with M_s <= L_s/128 + 1 and sum_s L_s^2 <= T * max_len
+    L.carry_slots_per_head = cdiv(T * max_len, 64) + 6 * T + 512 * B;
   }
   size_t off = 0;
   L.off_counts = off;      off = align_up(off + 256, 256);
@@ -61,9 +61,11 @@ int plan(const SbaArgs* a, Layout* out) {
 
 size_t elem_size(int dtype) { return dtype == SBA_F32 ? 4 : 2; }
 
-// A tensor is usable with 16-byte accesses when its base and its row/head/batch strides are 16-byte multiples.
-bool vec16(const SbaTensor& t, size_t es, bool fixed) {
+// A tensor is usable with 16-byte buffer accesses when its base and its row/head/batch strides are 16-byte
+// multiples and the rows of one sequence span less than 2 GiB (32-bit offsets from the sequence's first row).
+bool vec16(const SbaTensor& t, size_t es, bool fixed, int64_t max_rows) {
   const int64_t per = 16 / (int64_t)es;
+  if (max_rows * t.stride_token * (int64_t)es >= ((int64_t)1 << 31)) return false;
   if (((uintptr_t)t.ptr & 15) != 0) return false;
   if (t.stride_token % per || t.stride_head % per) return false;
   if (fixed && (t.stride_batch % per)) return false;
@@ -160,8 +162,9 @@ int sba_fwd(const SbaArgs* a) {
   p.head_dim = a->head_dim;
   p.scale_log2 = (float)((double)a->logit_scale * kLog2e);
   p.attend_current = a->attend_current ? 1 : 0;
+  const int64_t max_rows = (a->max_seqlen > 0 && a->max_seqlen < a->total_tokens) ? a->max_seqlen : a->total_tokens;
   bool v16 = (a->head_dim % (16 / (int)es)) == 0;
-  for (const SbaTensor* t : {&a->q, &a->k, &a->v}) v16 = v16 && vec16(*t, es, fixed);
+  for (const SbaTensor* t : {&a->q, &a->k, &a->v}) v16 = v16 && vec16(*t, es, fixed, max_rows);
   p.vec_ok = v16 ? 1 : 0;
   hipEvent_t* ev = (hipEvent_t*)a->trace_events;
   if (ev && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;
@@ -209,9 +212,10 @@ int sba_bwd(const SbaArgs* a) {
   p.scale_log2 = (float)((double)a->logit_scale * kLog2e);
   p.logit_scale = a->logit_scale;
   p.attend_current = a->attend_current ? 1 : 0;
+  const int64_t max_rows = (a->max_seqlen > 0 && a->max_seqlen < a->total_tokens) ? a->max_seqlen : a->total_tokens;
   bool v16 = (a->head_dim % (16 / (int)es)) == 0;
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
-    if (t->ptr) v16 = v16 && vec16(*t, es, fixed);
+    if (t->ptr) v16 = v16 && vec16(*t, es, fixed, max_rows);
   p.vec_ok = v16 ? 1 : 0;
   hipEvent_t* ev = (hipEvent_t*)a->trace_events;
   if (ev && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;

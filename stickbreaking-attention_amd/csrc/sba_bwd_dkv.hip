@@ -21,9 +21,7 @@ template <int DH> struct DkvLds {
   static constexpr int kPStride = lds_stride<kBlockK>();
   static constexpr int kQ = 0;
   static constexpr int kDo = kQ + kBlockQ * kRowStride;
-  static constexpr int kK = kDo + kBlockQ * kRowStride;
-  static constexpr int kV = kK + kBlockK * kRowStride;
-  static constexpr int kP = kV + kBlockK * kRowStride;
+  static constexpr int kP = kDo + kBlockQ * kRowStride;
   static constexpr int kDz = kP + kBlockQ * kPStride;
   static constexpr int kElems = kDz + kBlockQ * kPStride;
 };
@@ -39,8 +37,6 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
   T* lds = reinterpret_cast<T*>(lds_raw);
   T* q_lds = lds + Lds::kQ;
   T* do_lds = lds + Lds::kDo;
-  T* k_lds = lds + Lds::kK;
-  T* v_lds = lds + Lds::kV;
   T* p_lds = lds + Lds::kP;
   T* dz_lds = lds + Lds::kDz;
 
@@ -68,33 +64,44 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
 #pragma unroll
     for (int r = 0; r < 16; r++) { dkacc[b][r] = 0.f; dvacc[b][r] = 0.f; }
 
-  {
-    TileCopy<T, DH, kBlockK, kFast> ck, cv;
-    ck.load(kb + (int64_t)j0 * p.k.st, p.k.st, L - j0, D);
-    cv.load(vb + (int64_t)j0 * p.v.st, p.v.st, L - j0, D);
-    ck.store(k_lds);
-    cv.store(v_lds);
+  // This tile's K and V as MFMA A operands, stationary in registers: row tile mt, lane row l%32 -> key
+  // mfma_row_to_key(mt, l%32), 8 head_dim elements per k-step.  Keys beyond the sequence read as zero.
+  vec8 kf[2][kSteps], vf[2][kSteps];
+#pragma unroll
+  for (int mt = 0; mt < 2; mt++) {
+    const int key = j0 + mfma_row_to_key(mt, col);
+#pragma unroll
+    for (int kk = 0; kk < kSteps; kk++) {
+      kf[mt][kk] = as_vec8<T>(load_row8<T, kFast>(kb + (int64_t)key * p.k.st, 16 * kk + 8 * half, D, key < L));
+      vf[mt][kk] = as_vec8<T>(load_row8<T, kFast>(vb + (int64_t)key * p.v.st, 16 * kk + 8 * half, D, key < L));
+    }
   }
 
   const int first_row = j0 + 1 - ac;                                  // first row that sees key j0
   const int n_qt = (L + kBlockQ - 1) / kBlockQ;
   const int qt_begin = first_row < L ? first_row / kBlockQ : n_qt;    // == jt / 2 whenever any row sees the tile
-  const int64_t slot0 = (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] + carry_offset(jt, n_qt) -
-                        (int64_t)kBlockQ * (jt >> 1);      // + row
-  const float* carry = p.carry + slot0;
-  const float* prefix = p.prefix + slot0;
+  // product above the tile = above its upper 32-key sub-tile; prefix below the tile = below its lower sub-tile
+  const int64_t seq0 = (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] - (int64_t)kBlockQ * (jt >> 1);
+  const float* carry = p.carry + seq0 + carry_offset(2 * jt + 1, n_qt);      // + row
+  const float* prefix = p.prefix + seq0 + carry_offset(2 * jt, n_qt);
 
+  const RowSource<T> qsrc = make_row_source<T, kFast>(qb, p.q.st, L, D), dosrc = make_row_source<T, kFast>(dob, p.d_o.st, L, D);
+  TileCopy<T, DH, kBlockQ, kFast> cq, cdo;
+  if (qt_begin < n_qt) {
+    cq.load(qsrc, qt_begin * kBlockQ);
+    cdo.load(dosrc, qt_begin * kBlockQ);
+  }
   for (int qt = qt_begin; qt < n_qt; ++qt) {
     const int q0 = qt * kBlockQ;
-    __syncthreads();      // previous contraction finished reading q/do/p/dz tiles
-    {
-      TileCopy<T, DH, kBlockQ, kFast> cq;
-      cq.load(qb + (int64_t)q0 * p.q.st, p.q.st, L - q0, D);
-      cq.store(q_lds);
-      cq.load(dob + (int64_t)q0 * p.d_o.st, p.d_o.st, L - q0, D);
-      cq.store(do_lds);
-    }
+    __syncthreads();      // previous contraction finished reading the q/do/p/dz tiles
+    cq.store(q_lds);
+    cdo.store(do_lds);
     __syncthreads();
+    if (qt + 1 < n_qt) {  // prefetch the next query tile while this one is processed
+      const int qn = q0 + kBlockQ;
+      cq.load(qsrc, qn);
+      cdo.load(dosrc, qn);
+    }
 
     const int w_first = q0 + wave * 32, w_last = w_first + 31;
     const int qi = w_first + col;
@@ -115,23 +122,21 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
       for (int mt = 0; mt < 2; mt++) {
 #pragma unroll
         for (int r = 0; r < 16; r++) { s[mt][r] = 0.f; dp[mt][r] = 0.f; }
-        const int krow = mfma_row_to_key(mt, col);
 #pragma unroll
         for (int kk = 0; kk < kSteps; kk++) {
-          vec8 a = lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half);
           vec8 b = lds_row8<T>(q_lds, kRowStride, wave * 32 + col, 16 * kk + 8 * half);
-          s[mt] = Elem<T>::mfma(a, b, s[mt]);
+          s[mt] = Elem<T>::mfma(kf[mt][kk], b, s[mt]);
         }
 #pragma unroll
         for (int kk = 0; kk < kSteps; kk++) {
-          vec8 a = lds_row8<T>(v_lds, kRowStride, krow, 16 * kk + 8 * half);
           vec8 b = lds_row8<T>(do_lds, kRowStride, wave * 32 + col, 16 * kk + 8 * half);
-          dp[mt] = Elem<T>::mfma(a, b, dp[mt]);
+          dp[mt] = Elem<T>::mfma(vf[mt][kk], b, dp[mt]);
         }
       }
       const int lim = row_ok ? qi + ac - j0 - 32 * half : 0;
-      float prefix_next;
-      bwd_tile_math<T>(s, dp, p.scale_log2, diagonal, lim, half, drem, prod_in, prefix_in, pk, dzk, prefix_next);
+      float prod_lower, prefix_upper, prefix_next;
+      bwd_tile_math<T, 2>(s, dp, p.scale_log2, diagonal, lim, half, drem, prod_in, prefix_in, pk, dzk, prod_lower,
+                          prefix_upper, prefix_next);
     }
     // [query][key] tiles: this lane's 32 consecutive keys start at column 32*half of row 32*wave + col.
     {
@@ -178,6 +183,210 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// head_dim 128 fast path: producer / consumer waves.
+//
+// One workgroup = 8 waves = one 64-key tile, swept by query tiles of 64 rows.  Waves 0-3 are PRODUCERS: wave
+// (rg, g) takes rows 32*rg .. +31 against the 32-key sub-tile g (one MFMA row tile, 16 keys per lane, that
+// sub-tile's K/V operands stationary in registers), recomputes P^T and dZ^T and writes them to LDS.  Waves 4-7
+// are CONSUMERS: one step behind, wave cw contracts P^T/dZ^T with dO/Q over the 64 rows into the
+// 64-key x 32-column block cw of dV and dK.  Every SIMD hosts one producer (exp/rcp/VALU bound) and one consumer
+// (MFMA/LDS bound), so the two pipelines overlap, and there is ONE barrier per step: P/dZ are double-buffered
+// and Q/dO triple-buffered (written for step t+1, read by producers for step t and by consumers for step t-1).
+// The per-(row, sub-tile) carries are what the forward and the dQ kernel recorded at 32-key granularity.
+constexpr int kDkvRows = 64;      // query rows per step
+constexpr int kDkv3Threads = 512;
+template <int DH> struct Dkv3Lds {
+  static constexpr int kRowStride = lds_stride<DH>();
+  static constexpr int kPStride = lds_stride<kBlockK>();
+  static constexpr int kQdoTile = kDkvRows * kRowStride;     // one Q (or dO) tile
+  static constexpr int kPTile = kDkvRows * kPStride;         // one P (or dZ) tile
+  static constexpr int kQ = 0;                               // 3 buffers of {Q, dO}
+  static constexpr int kP = 6 * kQdoTile;                    // 2 buffers of {P, dZ}
+  static constexpr int kElems = kP + 4 * kPTile;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
+  constexpr int DH = 128;
+  typedef typename Elem<T>::vec8 vec8;
+  typedef Dkv3Lds<DH> Lds;
+  constexpr int kRowStride = Lds::kRowStride, kPStride = Lds::kPStride;
+  constexpr int kSteps = DH / 16;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+
+  int head, slot;
+  xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
+  if (slot >= p.counts[1]) return;
+  const Tile tile = p.k_tiles[slot];
+  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3;
+  const bool producer = threadIdx.x < 256;
+  const int half = lane >> 5, col = lane & 31;
+  const int L = tile.seq_len, j0 = tile.origin, ac = p.attend_current, D = DH;
+  const int64_t tok0 = tile.seq_start;
+  const int jt = j0 / kBlockK;
+
+  const int first_row = j0 + 1 - ac;                         // first row that sees key j0
+  const int n_qt = (L + kBlockQ - 1) / kBlockQ;
+  const int row_begin = first_row < L ? (first_row / kDkvRows) * kDkvRows : L;
+  const int n_steps = (L - row_begin + kDkvRows - 1) / kDkvRows;
+
+  if (producer) {
+    const int rg = wave >> 1, group = wave & 1;
+    const int jb = j0 + 32 * group;          // first key of this wave's sub-tile
+    const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
+    const T* kb = (const T*)p.k.ptr + tile.seq_id * p.k.sb + head * p.k.sh + tok0 * p.k.st;
+    const T* vb = (const T*)p.v.ptr + tile.seq_id * p.v.sb + head * p.v.sh + tok0 * p.v.st;
+    const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
+    const T* dremb = p.d_rem.ptr ? (const T*)p.d_rem.ptr + tile.seq_id * p.d_rem.sb + head * p.d_rem.sh + tok0 * p.d_rem.st : nullptr;
+    const int64_t slot0 = (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] +
+                          carry_offset(2 * jt + group, n_qt) - (int64_t)kBlockQ * (jt >> 1);      // + row
+    const float* carry = p.carry + slot0;
+    const float* prefix = p.prefix + slot0;
+
+    // This sub-tile's K and V as MFMA A operands, stationary in registers (keys beyond the sequence read as zero).
+    vec8 kf[kSteps], vf[kSteps];
+    {
+      const int key = jb + mfma_row_to_key32(col);
+#pragma unroll
+      for (int kk = 0; kk < kSteps; kk++) {
+        kf[kk] = as_vec8<T>(load_row8<T, true>(kb + (int64_t)key * p.k.st, 16 * kk + 8 * half, D, key < L));
+        vf[kk] = as_vec8<T>(load_row8<T, true>(vb + (int64_t)key * p.v.st, 16 * kk + 8 * half, D, key < L));
+      }
+    }
+    const RowSource<T> qsrc = make_row_source<T, true>(qb, p.q.st, L, D), dosrc = make_row_source<T, true>(dob, p.d_o.st, L, D);
+    TileCopy<T, DH, kDkvRows, true> cq, cdo;
+    if (n_steps > 0) {
+      cq.load(qsrc, row_begin);
+      cdo.load(dosrc, row_begin);
+      cq.store(lds + Lds::kQ);
+      cdo.store(lds + Lds::kQ + Lds::kQdoTile);
+      if (n_steps > 1) {
+        const int qn = row_begin + kDkvRows;
+        cq.load(qsrc, qn);
+        cdo.load(dosrc, qn);
+      }
+    }
+    __syncthreads();
+    for (int t = 0; t <= n_steps; ++t) {
+      if (t < n_steps) {
+        const int q0 = row_begin + t * kDkvRows;
+        const T* q_lds = lds + Lds::kQ + (t % 3) * 2 * Lds::kQdoTile;
+        const T* do_lds = q_lds + Lds::kQdoTile;
+        T* p_lds = lds + Lds::kP + (t & 1) * 2 * Lds::kPTile;
+        T* dz_lds = p_lds + Lds::kPTile;
+        const int w_first = q0 + rg * 32, w_last = w_first + 31;
+        const int qi = w_first + col;
+        const bool row_ok = qi < L;
+        uint32_t pk[8], dzk[8];
+        if (jb > w_last - 1 + ac || jb >= L) {
+#pragma unroll
+          for (int i = 0; i < 8; i++) { pk[i] = 0; dzk[i] = 0; }
+        } else {
+          const bool diagonal = (jb + 31) > (w_first - 1 + ac) || w_last >= L;
+          const float drem = (dremb && row_ok) ? (float)dremb[(int64_t)qi * p.d_rem.st] : 0.f;
+          const float prod_in = carry[qi], prefix_in = prefix[qi];
+          f32x16 s[1], dp[1];
+#pragma unroll
+          for (int r = 0; r < 16; r++) { s[0][r] = 0.f; dp[0][r] = 0.f; }
+#pragma unroll
+          for (int kk = 0; kk < kSteps; kk++) {
+            vec8 b = lds_row8<T>(q_lds, kRowStride, rg * 32 + col, 16 * kk + 8 * half);
+            s[0] = Elem<T>::mfma(kf[kk], b, s[0]);
+          }
+#pragma unroll
+          for (int kk = 0; kk < kSteps; kk++) {
+            vec8 b = lds_row8<T>(do_lds, kRowStride, rg * 32 + col, 16 * kk + 8 * half);
+            dp[0] = Elem<T>::mfma(vf[kk], b, dp[0]);
+          }
+          const int lim = row_ok ? qi + ac - jb - 16 * half : 0;
+          float prod_lower, prefix_upper, prefix_next;
+          bwd_tile_math<T, 1>(s, dp, p.scale_log2, diagonal, lim, half, drem, prod_in, prefix_in, pk, dzk, prod_lower,
+                              prefix_upper, prefix_next);
+        }
+        // [query][key] tiles: this lane's 16 consecutive keys start at column 32*group + 16*half of row 32*rg + col.
+        u32x4* pp = reinterpret_cast<u32x4*>(p_lds + (rg * 32 + col) * kPStride + 32 * group + 16 * half);
+        u32x4* dd = reinterpret_cast<u32x4*>(dz_lds + (rg * 32 + col) * kPStride + 32 * group + 16 * half);
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+          pp[c] = u32x4{pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
+          dd[c] = u32x4{dzk[4 * c], dzk[4 * c + 1], dzk[4 * c + 2], dzk[4 * c + 3]};
+        }
+        if (t + 1 < n_steps) {               // stage the next query tile, fetch the one after
+          T* nq_lds = lds + Lds::kQ + ((t + 1) % 3) * 2 * Lds::kQdoTile;
+          cq.store(nq_lds);
+          cdo.store(nq_lds + Lds::kQdoTile);
+          if (t + 2 < n_steps) {
+            const int qn = q0 + 2 * kDkvRows;
+            cq.load(qsrc, qn);
+            cdo.load(dosrc, qn);
+          }
+        }
+      }
+      __syncthreads();
+    }
+  } else {
+    // Output blocks of this consumer wave: both 32-key row tiles x head_dim columns 32*wave .. +31.
+    f32x16 dkacc[2], dvacc[2];
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) { dkacc[b][r] = 0.f; dvacc[b][r] = 0.f; }
+    __syncthreads();
+    for (int t = 0; t <= n_steps; ++t) {
+      if (t >= 1) {
+        const int u = t - 1;
+        const T* q_lds = lds + Lds::kQ + (u % 3) * 2 * Lds::kQdoTile;
+        const T* do_lds = q_lds + Lds::kQdoTile;
+        const T* p_lds = lds + Lds::kP + (u & 1) * 2 * Lds::kPTile;
+        const T* dz_lds = p_lds + Lds::kPTile;
+        // dV[key][d] += sum_i P[i][key] dO[i][d];  dK[key][d] += sum_i dZ[i][key] Q[i][d]   (i over the 64 rows)
+#pragma unroll
+        for (int c = 0; c < kDkvRows / 16; c++) {
+          const int row0 = 16 * c + 8 * half;
+          vec8 bd = lds_col8<T>(do_lds, kRowStride, row0, 32 * wave, lane);
+          vec8 bq = lds_col8<T>(q_lds, kRowStride, row0, 32 * wave, lane);
+#pragma unroll
+          for (int mt = 0; mt < 2; mt++) {
+            vec8 ap = lds_col8<T>(p_lds, kPStride, row0, 32 * mt, lane);
+            dvacc[mt] = Elem<T>::mfma(ap, bd, dvacc[mt]);
+            vec8 az = lds_col8<T>(dz_lds, kPStride, row0, 32 * mt, lane);
+            dkacc[mt] = Elem<T>::mfma(az, bq, dkacc[mt]);
+          }
+        }
+      }
+      __syncthreads();
+    }
+    // acc[mt][r]: key j0 + 32*mt + 8*(r/4) + 4*half + r%4, column 32*wave + col.
+    T* dkb = (T*)p.dk.ptr + tile.seq_id * p.dk.sb + head * p.dk.sh + tok0 * p.dk.st;
+    T* dvb = (T*)p.dv.ptr + tile.seq_id * p.dv.sb + head * p.dv.sh + tok0 * p.dv.st;
+    const int d = 32 * wave + col;
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int key = j0 + 32 * mt + 8 * (r >> 2) + 4 * half + (r & 3);
+        if (key < L) {
+          dkb[(int64_t)key * p.dk.st + d] = (T)(dkacc[mt][r] * p.logit_scale);
+          dvb[(int64_t)key * p.dv.st + d] = (T)dvacc[mt][r];
+        }
+      }
+  }
+}
+
+template <typename T>
+static hipError_t launch_dkv3(const BwdParams& p, int max_tiles, hipStream_t stream) {
+  const size_t lds_bytes = (size_t)Dkv3Lds<128>::kElems * sizeof(T);
+  // The tile set exceeds the default 64 KB dynamic-LDS cap; the attribute is per device and cheap to set.
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv3_kernel<T>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+  if (e != hipSuccess) return e;
+  const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kDkv3Threads);
+  hipLaunchKernelGGL((bwd_dkv3_kernel<T>), grid, block, lds_bytes, stream, p);
+  return hipGetLastError();
+}
+
 template <typename T, int DH, bool kFast>
 static hipError_t launch_one(const BwdParams& p, int max_tiles, hipStream_t stream) {
   const size_t lds_bytes = (size_t)DkvLds<DH>::kElems * sizeof(T);
@@ -192,7 +401,7 @@ static hipError_t launch_one(const BwdParams& p, int max_tiles, hipStream_t stre
 
 template <typename T>
 static hipError_t launch_t(const BwdParams& p, int max_tiles, hipStream_t stream) {
-  if (p.vec_ok && p.head_dim == 128) return launch_one<T, 128, true>(p, max_tiles, stream);
+  if (p.vec_ok && p.head_dim == 128) return launch_dkv3<T>(p, max_tiles, stream);
   if (p.vec_ok && p.head_dim == 64) return launch_one<T, 64, true>(p, max_tiles, stream);
   return p.head_dim <= 64 ? launch_one<T, 64, false>(p, max_tiles, stream) : launch_one<T, 128, false>(p, max_tiles, stream);
 }

@@ -70,10 +70,15 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
 #pragma unroll
     for (int r = 0; r < 16; r++) dqacc[dt][r] = 0.f;
 
+  // The forward's product above the next key tile (above its upper sub-tile), fetched one tile ahead.
+  auto carry_slot = [&](int t) { return carry_offset(2 * t + 1, n_qt) + (qi - kBlockQ * (t >> 1)); };
+  float n_prod = 1.f;
+  const RowSource<T> ksrc = make_row_source<T, kFast>(kb, p.k.st, L, D), vsrc = make_row_source<T, kFast>(vb, p.v.st, L, D);
   TileCopy<T, DH, kBlockK, kFast> ck, cv;
   if (n_kt > 0) {
-    ck.load(kb, p.k.st, L, D);
-    cv.load(vb, p.v.st, L, D);
+    ck.load(ksrc, 0);
+    cv.load(vsrc, 0);
+    n_prod = carry[carry_slot(0)];
   }
   for (int jt = 0; jt < n_kt; ++jt) {
     const int j0 = jt * kBlockK;
@@ -81,15 +86,21 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
     ck.store(k_lds);
     cv.store(v_lds);
     __syncthreads();
+    const float prod_in = n_prod;
     if (jt + 1 < n_kt) {
       const int jn = j0 + kBlockK;
-      ck.load(kb + (int64_t)jn * p.k.st, p.k.st, L - jn, D);
-      cv.load(vb + (int64_t)jn * p.v.st, p.v.st, L - jn, D);
+      ck.load(ksrc, jn);
+      cv.load(vsrc, jn);
+      n_prod = carry[carry_slot(jt + 1)];
     }
-    // For the key-stationary kernel: C just below this tile, for every row of the tile.
-    const int64_t slot_idx = carry_offset(jt, n_qt) + (qi - kBlockQ * (jt >> 1));
-    if (half == 0) prefix_out[slot_idx] = prefix;
-    if (j0 > w_last - 1 + ac) continue;
+    // For the key-stationary kernel: C just below each 32-key sub-tile, for every row of the tile.
+    const int64_t slot_lo = carry_offset(2 * jt, n_qt) + (qi - kBlockQ * (jt >> 1));
+    const int64_t slot_hi = carry_offset(2 * jt + 1, n_qt) + (qi - kBlockQ * (jt >> 1));
+    if (half == 0) prefix_out[slot_lo] = prefix;
+    if (j0 > w_last - 1 + ac) {
+      if (half == 0) prefix_out[slot_hi] = prefix;
+      continue;
+    }
     const bool diagonal = (j0 + kBlockK - 1) > (w_first - 1 + ac) || w_last >= L;
 
     f32x16 s[2], dp[2];
@@ -111,7 +122,10 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
     }
     const int lim = row_ok ? qi + ac - j0 - 32 * half : 0;
     uint32_t pk[16], dzk[16];
-    bwd_tile_math<T>(s, dp, p.scale_log2, diagonal, lim, half, drem, carry[slot_idx], prefix, pk, dzk, prefix);
+    float prod_lower, prefix_upper;
+    bwd_tile_math<T, 2>(s, dp, p.scale_log2, diagonal, lim, half, drem, prod_in, prefix, pk, dzk, prod_lower,
+                        prefix_upper, prefix);
+    if (half == 0) prefix_out[slot_hi] = prefix_upper;
 
     // dQ += dZ K: A = dZ from registers, B = K gathered down the keys.
 #pragma unroll

@@ -119,35 +119,60 @@ __device__ __forceinline__ typename Elem<T>::vec8 lds_col8(const T* tile, int ro
 __device__ __forceinline__ int mfma_row_to_key(int mt, int m) {
   return ((m >> 2) & 1) * 32 + mt * 16 + (m >> 3) * 4 + (m & 3);
 }
+// Same for a 32-key sub-tile handled as ONE row tile: register r of half-wave h holds key 16*h + r.
+__device__ __forceinline__ int mfma_row_to_key32(int m) { return ((m >> 2) & 1) * 16 + (m >> 3) * 4 + (m & 3); }
+
+// The rows of one (head, sequence) of a [.., token, head_dim] tensor, as the tile copies see them.  The fast path
+// addresses them through a raw buffer resource: scalar base, out-of-range rows read as zero for free, and one
+// loop-invariant 32-bit lane offset instead of 64-bit pointer arithmetic per chunk.
+template <typename T>
+struct RowSource {
+  const T* base;
+  int64_t stride;                 // elements between token rows
+  int rows, d;                    // valid rows, valid head_dim
+  __amdgpu_buffer_rsrc_t rsrc;    // base .. last valid element (fast path only)
+  int stride_bytes;
+};
+template <typename T, bool kFast>
+__device__ __forceinline__ RowSource<T> make_row_source(const T* base, int64_t stride, int rows, int d) {
+  RowSource<T> r;
+  r.base = base; r.stride = stride; r.rows = rows; r.d = d;
+  r.stride_bytes = (int)(stride * (int64_t)sizeof(T));
+  if (kFast) {
+    const int bytes = rows > 0 ? (rows - 1) * r.stride_bytes + d * (int)sizeof(T) : 0;
+    r.rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
+  }
+  return r;
+}
 
 // Cooperative global -> register -> LDS copy of a [kRows x DH] tile of 16-bit elements, 16 bytes per access.
-// kFast: head_dim == DH and every row start is 16-byte aligned, so the copy is straight-line 16-byte loads.
-// Otherwise rows at or beyond `rows_valid` (>= 1) and columns at or beyond `d_valid` are zero-filled.
-template <typename T, int DH, int kRows, bool kFast>
+// Rows beyond the source and columns at or beyond head_dim are zero-filled.  kFast: head_dim == DH, every row
+// start 16-byte aligned and the sequence's rows span < 2 GiB, so the copy is straight-line buffer loads.
+template <typename T, int DH, int kRows, bool kFast, int kNumThreads = kThreads>
 struct TileCopy {
   static constexpr int kChunksPerRow = DH / 8;
-  static constexpr int kChunks = kRows * kChunksPerRow;
-  static constexpr int kPerThread = kChunks / kThreads;
-  static_assert(kChunks % kThreads == 0, "tile must divide evenly over the workgroup");
+  static constexpr int kRowsPerPass = kNumThreads / kChunksPerRow;
+  static constexpr int kPerThread = kRows / kRowsPerPass;
+  static_assert(kRows % kRowsPerPass == 0, "tile must divide evenly over the workgroup");
   u32x4 regs[kPerThread];
 
-  __device__ __forceinline__ void load(const T* base, int64_t row_stride, int rows_valid, int d_valid) {
+  __device__ __forceinline__ void load(const RowSource<T>& src, int row0) {
+    const int tr = (threadIdx.x % kNumThreads) / kChunksPerRow, col = ((threadIdx.x % kNumThreads) % kChunksPerRow) * 8;
+    if (kFast) {
+      const int voff = tr * src.stride_bytes + col * (int)sizeof(T);
 #pragma unroll
-    for (int i = 0; i < kPerThread; i++) {
-      const int c = threadIdx.x + i * kThreads;
-      const int row = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
-      if (kFast) {
-        // Out-of-range rows re-read the last valid row: finite data that every consumer masks (a key beyond the
-        // sequence is hidden from every row; a query row beyond it is forced hidden) -- no zero fill needed.
-        const int rr = min(row, rows_valid - 1);
-        regs[i] = *reinterpret_cast<const u32x4*>(base + rr * row_stride + col);
-      } else {
+      for (int i = 0; i < kPerThread; i++)
+        regs[i] = __builtin_amdgcn_raw_buffer_load_b128(src.rsrc, voff, (row0 + i * kRowsPerPass) * src.stride_bytes, 0);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kPerThread; i++) {
+        const int row = row0 + tr + i * kRowsPerPass;
         u32x4 v = {0, 0, 0, 0};
-        if (row < rows_valid) {
-          const uint16_t* p = reinterpret_cast<const uint16_t*>(base + row * row_stride + col);
+        if (row < src.rows) {
+          const uint16_t* p = reinterpret_cast<const uint16_t*>(src.base + row * src.stride + col);
           uint16_t e[8];
 #pragma unroll
-          for (int t = 0; t < 8; t++) e[t] = (col + t < d_valid) ? p[t] : (uint16_t)0;
+          for (int t = 0; t < 8; t++) e[t] = (col + t < src.d) ? p[t] : (uint16_t)0;
           v[0] = e[0] | ((uint32_t)e[1] << 16); v[1] = e[2] | ((uint32_t)e[3] << 16);
           v[2] = e[4] | ((uint32_t)e[5] << 16); v[3] = e[6] | ((uint32_t)e[7] << 16);
         }
@@ -156,12 +181,10 @@ struct TileCopy {
     }
   }
   __device__ __forceinline__ void store(T* tile) const {
+    const int tr = (threadIdx.x % kNumThreads) / kChunksPerRow, col = ((threadIdx.x % kNumThreads) % kChunksPerRow) * 8;
 #pragma unroll
-    for (int i = 0; i < kPerThread; i++) {
-      const int c = threadIdx.x + i * kThreads;
-      const int row = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
-      *reinterpret_cast<u32x4*>(tile + row * lds_stride<DH>() + col) = regs[i];
-    }
+    for (int i = 0; i < kPerThread; i++)
+      *reinterpret_cast<u32x4*>(tile + (tr + i * kRowsPerPass) * lds_stride<DH>() + col) = regs[i];
   }
 };
 
@@ -188,22 +211,26 @@ constexpr float kExpClamp = 100.0f;   // 2^100 and 2^-100 are finite; sigma(z) i
 // Element-wise backward math of one 64-key tile for the 32 keys this lane owns (see the conventions above).
 //   s, dp     : S^T = K Q^T and dP^T = V dO^T accumulators (row tile mt, register r  <->  key 32*half + 16*mt + r)
 //   lim       : key R of this lane is visible iff R < lim (only consulted when `diagonal`)
+//   NT        : MFMA row tiles per key tile: 2 for a 64-key tile (keys 32*half + 16*mt + r), 1 for a 32-key
+//               sub-tile (keys 16*half + r)
 //   prod_in   : prod over the keys ABOVE this tile (between the tile and the row) of (1 - sigma); recorded by
 //               the forward, which sweeps in that direction
 //   prefix_in : sum over the keys BELOW this tile of g, with g_ij = A_ij (dO_i.v_j - drem_i)
 // Produces P (pk) and dZ = g - sigma * C (dzk), C_ij = sum_{j' <= j} g_ij', packed to 16 bit two keys per
 // word, and the prefix sum for the next tile up.  (The reference evaluates the same quantities tile by tile at
 // stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:438-447.)
-template <typename T, bool kDiagonal>
-__device__ __forceinline__ void bwd_tile_math_impl(const f32x16 (&s)[2], const f32x16 (&dp)[2], float scale_log2, int lim,
+template <typename T, int NT, bool kDiagonal>
+__device__ __forceinline__ void bwd_tile_math_impl(const f32x16 (&s)[NT], const f32x16 (&dp)[NT], float scale_log2, int lim,
                                                    int half, float drem, float prod_in, float prefix_in,
-                                                   uint32_t (&pk)[16], uint32_t (&dzk)[16], float& prefix_out) {
+                                                   uint32_t (&pk)[8 * NT], uint32_t (&dzk)[8 * NT], float& prod_lower,
+                                                   float& prefix_upper, float& prefix_out) {
+  constexpr int N = 16 * NT;      // keys per lane
   // sigma = 1 - 1/(1+e) needs no clamp on e: e = inf gives 1/(1+e) = 0 and sigma = 1 exactly, and the absolute
   // error of the subtraction (6e-8) is far below the 16-bit rounding of P and dZ.
-  float beta[32], pe[32];
+  float beta[N], pe[N];
   float run = 1.f;
 #pragma unroll
-  for (int R = 31; R >= 0; --R) {
+  for (int R = N - 1; R >= 0; --R) {
     float x = s[R >> 4][R & 15] * scale_log2;
     if (kDiagonal) x = (R < lim) ? x : -INFINITY;
     const float omb = fast_rcp(1.f + fast_exp2(x));
@@ -212,13 +239,14 @@ __device__ __forceinline__ void bwd_tile_math_impl(const f32x16 (&s)[2], const f
     run *= omb;
   }
   const float oth = other_half(run, half);
-  const float seed = half ? prod_in : prod_in * oth;      // the upper half-wave holds the higher keys
+  prod_lower = prod_in * (half ? run : oth);               // product above the lower half-wave's keys
+  const float seed = half ? prod_in : prod_lower;           // the upper half-wave holds the higher keys
   // Running C as if this lane's keys were preceded only by the keys below the tile; the upper half-wave's
   // share of the lower half-wave's total is added afterwards (fixup).
   float acc = prefix_in;
-  float dz[32];
+  float dz[N];
 #pragma unroll
-  for (int R = 0; R < 32; R++) {
+  for (int R = 0; R < N; R++) {
     const float a = beta[R] * (pe[R] * seed);
     const float g = a * (dp[R >> 4][R & 15] - drem);
     acc += g;
@@ -228,22 +256,28 @@ __device__ __forceinline__ void bwd_tile_math_impl(const f32x16 (&s)[2], const f
   const float tot = acc - prefix_in;
   const float oth_g = other_half(tot, half);
   const float fixup = half ? oth_g : 0.f;                   // the lower half-wave holds the lower keys
+  prefix_upper = prefix_in + (half ? oth_g : tot);          // C just below the upper half-wave's keys
   prefix_out = acc + oth_g;
 #pragma unroll
-  for (int R = 0; R < 32; R += 2) {
+  for (int R = 0; R < N; R += 2) {
     pk[R >> 1] = pack2<T>(pe[R], pe[R + 1]);
     dzk[R >> 1] = pack2<T>(dz[R] - beta[R] * fixup, dz[R + 1] - beta[R + 1] * fixup);
   }
 }
 
-template <typename T>
-__device__ __forceinline__ void bwd_tile_math(const f32x16 (&s)[2], const f32x16 (&dp)[2], float scale_log2, bool diagonal,
+// prod_lower / prefix_upper: the same two carries at the boundary between the two half-waves' keys (the middle of
+// the tile), for consumers that work on half the keys at a time.
+template <typename T, int NT>
+__device__ __forceinline__ void bwd_tile_math(const f32x16 (&s)[NT], const f32x16 (&dp)[NT], float scale_log2, bool diagonal,
                                               int lim, int half, float drem, float prod_in, float prefix_in,
-                                              uint32_t (&pk)[16], uint32_t (&dzk)[16], float& prefix_out) {
+                                              uint32_t (&pk)[8 * NT], uint32_t (&dzk)[8 * NT], float& prod_lower,
+                                              float& prefix_upper, float& prefix_out) {
   if (diagonal)
-    bwd_tile_math_impl<T, true>(s, dp, scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prefix_out);
+    bwd_tile_math_impl<T, NT, true>(s, dp, scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prod_lower,
+                                    prefix_upper, prefix_out);
   else
-    bwd_tile_math_impl<T, false>(s, dp, scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prefix_out);
+    bwd_tile_math_impl<T, NT, false>(s, dp, scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prod_lower,
+                                     prefix_upper, prefix_out);
 }
 
 // Map the linear workgroup id to (head, tile slot) so that the workgroups of one head land on one XCD

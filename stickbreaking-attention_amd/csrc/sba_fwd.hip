@@ -57,11 +57,11 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FwdParams p) {
   const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
   float* carry = p.carry ? p.carry + (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] : nullptr;
 
+  const RowSource<T> ksrc = make_row_source<T, kFast>(kb, p.k.st, L, D), vsrc = make_row_source<T, kFast>(vb, p.v.st, L, D);
   TileCopy<T, DH, kBlockK, kFast> ck, cv;
   if (n_kt > 0) {
-    const int j0 = (n_kt - 1) * kBlockK;
-    ck.load(kb + (int64_t)j0 * p.k.st, p.k.st, L - j0, D);
-    cv.load(vb + (int64_t)j0 * p.v.st, p.v.st, L - j0, D);
+    ck.load(ksrc, (n_kt - 1) * kBlockK);
+    cv.load(vsrc, (n_kt - 1) * kBlockK);
   }
   for (int jt = n_kt - 1; jt >= 0; --jt) {
     const int j0 = jt * kBlockK;
@@ -71,12 +71,17 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FwdParams p) {
     __syncthreads();
     if (jt > 0) {
       const int jn = j0 - kBlockK;
-      ck.load(kb + (int64_t)jn * p.k.st, p.k.st, L - jn, D);
-      cv.load(vb + (int64_t)jn * p.v.st, p.v.st, L - jn, D);
+      ck.load(ksrc, jn);
+      cv.load(vsrc, jn);
     }
-    // For the backward: the product over the keys between this tile and the row, for every row of the tile.
-    if (carry && half == 0) carry[carry_offset(jt, n_qt) + (qi - kBlockQ * (jt >> 1))] = prod;
-    if (j0 > w_last - 1 + ac) continue;                       // nothing visible to this wave yet
+    // For the backward: the product over the keys between the upper 32-key sub-tile and the row, for every row
+    // of the tile (the lower sub-tile's value follows once this tile's upper half is known).
+    const int64_t cslot = qi - kBlockQ * (jt >> 1);
+    if (carry && half == 0) carry[carry_offset(2 * jt + 1, n_qt) + cslot] = prod;
+    if (j0 > w_last - 1 + ac) {                               // nothing visible to this wave yet
+      if (carry && half == 0) carry[carry_offset(2 * jt, n_qt) + cslot] = prod;
+      continue;
+    }
     const bool diagonal = (j0 + kBlockK - 1) > (w_first - 1 + ac);
 
     // S^T tile: rows = keys (permuted so that a lane ends up with 32 consecutive keys), columns = queries.
@@ -119,6 +124,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FwdParams p) {
     const float oth = other_half(run, half);
     // The upper half-wave holds the higher keys, which come first in the sweep.
     const float seed = half ? prod : prod * oth;
+    if (carry && half == 0) carry[carry_offset(2 * jt, n_qt) + cslot] = seed;   // product above the lower sub-tile
     prod = (prod * oth) * run;
 
     // O += P V: A = P from registers (k index <-> key 32*half + 8c + t), B = V gathered down the keys.

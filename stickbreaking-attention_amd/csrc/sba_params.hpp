@@ -58,8 +58,8 @@ struct BwdParams {
   const Tile* k_tiles;
   const int32_t* counts;
   const int64_t* carry_base;
-  const float* carry;          // [head][slot]: the forward's running product per (row, key tile)
-  float* prefix;               // [head][slot]: prefix sum of g over the keys below the tile, per (row, key tile)
+  const float* carry;          // [head][slot]: the forward's running product per (row, 32-key sub-tile)
+  float* prefix;               // [head][slot]: prefix sum of g over the keys below the sub-tile, per (row, sub-tile)
   int64_t carry_head_stride;   // carry slots reserved per head
   int32_t num_heads, head_dim;
   float scale_log2;
@@ -68,14 +68,15 @@ struct BwdParams {
   int32_t vec_ok;
 };
 
-// Carry slots of one sequence whose length rounds up to M query tiles: key tiles 2m and 2m+1 are needed
-// by the rows of query tiles m, m+1, ..., M-1.  Slot of (key tile J, row i), i >= 128*(J/2):
-//   carry_offset(J, M) + (i - 128*(J/2))
-__host__ __device__ inline int64_t carry_offset(int64_t J, int64_t M) {
-  const int64_t m = J >> 1;
-  const int64_t tri = (J & 1) ? m * m : m * (m - 1);      // sum_{J' < J} floor(J'/2)
-  return J * (M * 128) - 128 * tri;
+// Carry slots.  Carries are kept per (row, 32-key sub-tile): sub-tile U covers keys 32U .. 32U+31 of the
+// sequence and is needed by the rows of query tiles U/4, U/4 + 1, ..., M-1 (M = query tiles of 128 rows the
+// sequence rounds up to).  Slot of (sub-tile U, row i), i >= 128*(U/4):
+//   carry_offset(U, M) + (i - 128*(U/4))
+__host__ __device__ inline int64_t carry_offset(int64_t U, int64_t M) {
+  const int64_t q = U >> 2, r = U & 3;
+  const int64_t tri = 2 * q * (q - 1) + r * q;            // sum_{U' < U} floor(U'/4)
+  return U * (M * 128) - 128 * tri;
 }
-__host__ __device__ inline int64_t carry_slots(int64_t M) { return 128 * M * (M + 1); }   // carry_offset(2M, M)
+__host__ __device__ inline int64_t carry_slots(int64_t M) { return 256 * M * (M + 1); }   // carry_offset(4M, M)
 
 }  // namespace sba

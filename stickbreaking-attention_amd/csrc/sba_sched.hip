@@ -2,16 +2,18 @@
 //
 // The reference pads every sequence to the longest one: its grid is (num_seqs, H/2, max_len/64 + 1) programs,
 // most of which exit idle on a ragged batch (stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:475-479, :294).
-// Here a single small kernel reads cu_seqlens on the device (no host synchronisation), enumerates exactly the
-// tiles that exist and orders them heaviest first (a query tile that starts at row q0 sweeps ~q0/64 key
-// tiles), so the one launch that follows fills the chip without padding and ends with the cheap tiles.
-// It also lays out the backward's per-(row, key tile) carries contiguously per sequence.
+// Here a single small kernel reads cu_seqlens on the device (no host synchronisation) and enumerates exactly the
+// tiles that exist, so the one launch that follows fills the chip without padding.  Order: sequences longest
+// first, and inside a sequence the heaviest tile first (the last query tile / the first key tile).  The tiles of
+// one (head, sequence) are therefore resident together and sweep the same K/V (or Q/dO) rows a step or two apart,
+// which keeps those rows in the XCD's L2 instead of re-fetching them from HBM, and the launch still ends with
+// the cheap tiles of the short sequences.  It also lays out the per-(row, 32-key sub-tile) carries per sequence.
 #include "sba_device.hpp"
 #include "sba_params.hpp"
 
 namespace sba {
 
-constexpr int kBins = 4096;          // work histogram bins (work = number of tiles swept, saturating)
+constexpr int kBins = 4096;          // sequence length classes (query tiles per sequence, saturating)
 constexpr int kSchedThreads = 1024;
 
 __device__ __forceinline__ int64_t read_cu(const SchedParams& p, int idx) {
@@ -69,37 +71,40 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
   if (threadIdx.x == 0) carry_run = 0;
   __syncthreads();
 
-  // Pass 1: histogram of tile work.  One wave per sequence, lanes stride over its tiles.
-  for (int s = wave; s < p.num_seqs; s += nwaves) {
+  // Pass 1: tiles per length class (class = number of query tiles of the sequence, saturating).
+  for (int s = threadIdx.x; s < p.num_seqs; s += kSchedThreads) {
     int start, len;
     seq_bounds(p, s, &start, &len);
-    const int nq = (len + kBlockQ - 1) / kBlockQ;
-    for (int t = lane; t < nq; t += 64) atomicAdd(&qbins[min(q_tile_work(t * kBlockQ, len, p.attend_current), kBins - 1)], 1);
-    if (p.want_key_tiles) {
-      const int nk = (len + kBlockK - 1) / kBlockK;
-      for (int t = lane; t < nk; t += 64) atomicAdd(&kbins[min(k_tile_work(t * kBlockK, len, p.attend_current), kBins - 1)], 1);
-    }
+    const int nq = (len + kBlockQ - 1) / kBlockQ, nk = (len + kBlockK - 1) / kBlockK;
+    const int cls = min(nq, kBins - 1);
+    if (nq) atomicAdd(&qbins[cls], nq);
+    if (nk && p.want_key_tiles) atomicAdd(&kbins[cls], nk);
   }
   __syncthreads();
   descending_offsets(qbins, scratch);
   if (p.want_key_tiles) descending_offsets(kbins, scratch);
 
-  // Pass 2: scatter the descriptors.
+  // Pass 2: each sequence takes a contiguous range of slots in its class; one wave per sequence.
   for (int s = wave; s < p.num_seqs; s += nwaves) {
     int start, len;
     seq_bounds(p, s, &start, &len);
-    const int nq = (len + kBlockQ - 1) / kBlockQ;
-    for (int t = lane; t < nq; t += 64) {
-      const int pos = atomicAdd(&qbins[min(q_tile_work(t * kBlockQ, len, p.attend_current), kBins - 1)], 1);
-      Tile d; d.seq_start = start; d.seq_len = len; d.origin = t * kBlockQ; d.seq_id = s;
-      p.q_tiles[pos] = d;
+    const int nq = (len + kBlockQ - 1) / kBlockQ, nk = (len + kBlockK - 1) / kBlockK;
+    const int cls = min(nq, kBins - 1);
+    int qbase = 0, kbase = 0;
+    if (lane == 0) {
+      if (nq) qbase = atomicAdd(&qbins[cls], nq);
+      if (nk && p.want_key_tiles) kbase = atomicAdd(&kbins[cls], nk);
+    }
+    qbase = __shfl(qbase, 0);
+    kbase = __shfl(kbase, 0);
+    for (int t = lane; t < nq; t += 64) {        // heaviest query tile (the last one) first
+      Tile d; d.seq_start = start; d.seq_len = len; d.origin = (nq - 1 - t) * kBlockQ; d.seq_id = s;
+      p.q_tiles[qbase + t] = d;
     }
     if (p.want_key_tiles) {
-      const int nk = (len + kBlockK - 1) / kBlockK;
-      for (int t = lane; t < nk; t += 64) {
-        const int pos = atomicAdd(&kbins[min(k_tile_work(t * kBlockK, len, p.attend_current), kBins - 1)], 1);
+      for (int t = lane; t < nk; t += 64) {      // heaviest key tile (the first one) first
         Tile d; d.seq_start = start; d.seq_len = len; d.origin = t * kBlockK; d.seq_id = s;
-        p.k_tiles[pos] = d;
+        p.k_tiles[kbase + t] = d;
       }
     }
   }

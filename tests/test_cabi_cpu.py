@@ -63,14 +63,15 @@ def _args(native, H, D, T, B, varlen=True, max_seqlen=0, dtype=0):
 
 def test_workspace_sizes_cover_any_batch(native):
     """The carry buffer is sized from (T, max_seqlen, num_seqs) alone; it must cover the exact need
-    sum_s 128 M_s (M_s + 1), M_s = ceil(L_s / 128), of every batch with those totals."""
+    sum_s 256 M_s (M_s + 1), M_s = ceil(L_s / 128), of every batch with those totals (one fp32 per row and
+    32-key sub-tile the row sweeps)."""
     lib = native.lib()
     rng = np.random.default_rng(0)
     for _ in range(200):
         B = int(rng.integers(1, 40))
         lengths = rng.integers(1, int(rng.choice([4, 70, 300, 5000])), size=B)
         T, mx, H = int(lengths.sum()), int(lengths.max()), int(rng.integers(1, 9))
-        need = sum(128 * m * (m + 1) for m in (-(-int(n) // 128) for n in lengths)) * H * 4
+        need = sum(256 * m * (m + 1) for m in (-(-int(n) // 128) for n in lengths)) * H * 4
         fwd, bwd, carry = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
         for hint in (mx, 0):
             a = _args(native, H, 64, T, B, max_seqlen=hint)
@@ -80,7 +81,7 @@ def test_workspace_sizes_cover_any_batch(native):
     # fixed-length mode is exact
     a = _args(native, 3, 128, 500, 4, varlen=False)
     assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, ctypes.byref(carry)) == 0
-    assert carry.value == -(-(4 * 128 * 4 * 5 * 3 * 4) // 256) * 256
+    assert carry.value == -(-(4 * 256 * 4 * 5 * 3 * 4) // 256) * 256
 
 
 def test_size_query_validates(native):
