@@ -256,8 +256,20 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
       }
     }
     const RowSource<T> qsrc = make_row_source<T, true>(qb, p.q.st, L, D), dosrc = make_row_source<T, true>(dob, p.d_o.st, L, D);
+    // Per-row scalars (drem, product above the sub-tile, C below it) are fetched one step ahead and BEFORE the
+    // tile prefetch of that step: memory results return in order, so a scalar consumed right after a younger
+    // tile load was issued would drain the whole prefetch.
+    T n_drem = (T)0.f;
+    float n_prod = 1.f, n_prefix = 0.f;
+    auto fetch_row_scalars = [&](int row0) {
+      const int r = row0 + rg * 32 + col;
+      n_drem = (dremb && r < L) ? dremb[(int64_t)r * p.d_rem.st] : (T)0.f;
+      n_prod = carry[r];
+      n_prefix = prefix[r];
+    };
     TileCopy<T, DH, kDkvRows, true> cq, cdo;
     if (n_steps > 0) {
+      fetch_row_scalars(row_begin);
       cq.load(qsrc, row_begin);
       cdo.load(dosrc, row_begin);
       cq.store(lds + Lds::kQ);
@@ -276,6 +288,20 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
         const T* do_lds = q_lds + Lds::kQdoTile;
         T* p_lds = lds + Lds::kP + (t & 1) * 2 * Lds::kPTile;
         T* dz_lds = p_lds + Lds::kPTile;
+        // Stage the next query tile (fetched during the previous step) and start fetching the one after; the
+        // barrier that ends this step is the only point that waits for these loads.
+        const float drem = (float)n_drem, prod_in = n_prod, prefix_in = n_prefix;
+        if (t + 1 < n_steps) fetch_row_scalars(q0 + kDkvRows);
+        if (t + 1 < n_steps) {
+          T* nq_lds = lds + Lds::kQ + ((t + 1) % 3) * 2 * Lds::kQdoTile;
+          cq.store(nq_lds);
+          cdo.store(nq_lds + Lds::kQdoTile);
+          if (t + 2 < n_steps) {
+            const int qn = q0 + 2 * kDkvRows;
+            cq.load(qsrc, qn);
+            cdo.load(dosrc, qn);
+          }
+        }
         const int w_first = q0 + rg * 32, w_last = w_first + 31;
         const int qi = w_first + col;
         const bool row_ok = qi < L;
@@ -285,20 +311,22 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
           for (int i = 0; i < 8; i++) { pk[i] = 0; dzk[i] = 0; }
         } else {
           const bool diagonal = (jb + 31) > (w_first - 1 + ac) || w_last >= L;
-          const float drem = (dremb && row_ok) ? (float)dremb[(int64_t)qi * p.d_rem.st] : 0.f;
-          const float prod_in = carry[qi], prefix_in = prefix[qi];
           f32x16 s[1], dp[1];
 #pragma unroll
           for (int r = 0; r < 16; r++) { s[0][r] = 0.f; dp[0][r] = 0.f; }
+          // All sixteen B operands are requested before the first MFMA: the consumers keep the LDS queue long,
+          // and a read-two / wait / multiply-two schedule pays that queueing latency eight times over.
+          vec8 bq[kSteps], bdo[kSteps];
 #pragma unroll
           for (int kk = 0; kk < kSteps; kk++) {
-            vec8 b = lds_row8<T>(q_lds, kRowStride, rg * 32 + col, 16 * kk + 8 * half);
-            s[0] = Elem<T>::mfma(kf[kk], b, s[0]);
+            bq[kk] = lds_row8<T>(q_lds, kRowStride, rg * 32 + col, 16 * kk + 8 * half);
+            bdo[kk] = lds_row8<T>(do_lds, kRowStride, rg * 32 + col, 16 * kk + 8 * half);
           }
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int kk = 0; kk < kSteps; kk++) {
-            vec8 b = lds_row8<T>(do_lds, kRowStride, rg * 32 + col, 16 * kk + 8 * half);
-            dp[0] = Elem<T>::mfma(vf[kk], b, dp[0]);
+            s[0] = Elem<T>::mfma(kf[kk], bq[kk], s[0]);
+            dp[0] = Elem<T>::mfma(vf[kk], bdo[kk], dp[0]);
           }
           const int lim = row_ok ? qi + ac - jb - 16 * half : 0;
           float prod_lower, prefix_upper, prefix_next;
@@ -312,16 +340,6 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
         for (int c = 0; c < 2; c++) {
           pp[c] = u32x4{pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
           dd[c] = u32x4{dzk[4 * c], dzk[4 * c + 1], dzk[4 * c + 2], dzk[4 * c + 3]};
-        }
-        if (t + 1 < n_steps) {               // stage the next query tile, fetch the one after
-          T* nq_lds = lds + Lds::kQ + ((t + 1) % 3) * 2 * Lds::kQdoTile;
-          cq.store(nq_lds);
-          cdo.store(nq_lds + Lds::kQdoTile);
-          if (t + 2 < n_steps) {
-            const int qn = q0 + 2 * kDkvRows;
-            cq.load(qsrc, qn);
-            cdo.load(dosrc, qn);
-          }
         }
       }
       __syncthreads();

@@ -19,14 +19,15 @@
 
 namespace sba {
 
-template <typename T, int DH, bool kFast>
-__global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
+template <typename T, int DH, bool kFast, int KT>
+__global__ __launch_bounds__(kThreads, KT == 32 ? 2 : 1) void bwd_dq_kernel(BwdParams p) {
+  constexpr int NT = KT / 32;         // MFMA row tiles per key tile: a lane owns 16*NT consecutive keys
   typedef typename Elem<T>::vec8 vec8;
   constexpr int kRowStride = lds_stride<DH>();
   constexpr int kSteps = DH / 16;
   constexpr int kDTiles = DH / 32;
-  __shared__ __attribute__((aligned(16))) T k_lds[kBlockK * kRowStride];
-  __shared__ __attribute__((aligned(16))) T v_lds[kBlockK * kRowStride];
+  __shared__ __attribute__((aligned(16))) T k_lds[KT * kRowStride];
+  __shared__ __attribute__((aligned(16))) T v_lds[KT * kRowStride];
 
   int head, slot;
   xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
@@ -57,7 +58,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
 
   const int last_row = min(q0 + kBlockQ, L) - 1;
   const int last_key = last_row - 1 + ac;
-  const int n_kt = last_key < 0 ? 0 : last_key / kBlockK + 1;
+  const int n_kt = last_key < 0 ? 0 : last_key / KT + 1;
   const int w_first = q0 + wave * 32, w_last = w_first + 31;
   const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
   const int64_t slot0 = (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id];
@@ -71,44 +72,49 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
     for (int r = 0; r < 16; r++) dqacc[dt][r] = 0.f;
 
   // The forward's product above the next key tile (above its upper sub-tile), fetched one tile ahead.
-  auto carry_slot = [&](int t) { return carry_offset(2 * t + 1, n_qt) + (qi - kBlockQ * (t >> 1)); };
+  // sub-tile whose upper edge is the upper edge of key tile t, and the first row that owns slots for tile t
+  auto carry_slot = [&](int t) {
+    const int u = NT == 2 ? 2 * t + 1 : t;
+    return carry_offset(u, n_qt) + (qi - kBlockQ * (u >> 2));
+  };
   float n_prod = 1.f;
   const RowSource<T> ksrc = make_row_source<T, kFast>(kb, p.k.st, L, D), vsrc = make_row_source<T, kFast>(vb, p.v.st, L, D);
-  TileCopy<T, DH, kBlockK, kFast> ck, cv;
+  TileCopy<T, DH, KT, kFast> ck, cv;
   if (n_kt > 0) {
     ck.load(ksrc, 0);
     cv.load(vsrc, 0);
     n_prod = carry[carry_slot(0)];
   }
   for (int jt = 0; jt < n_kt; ++jt) {
-    const int j0 = jt * kBlockK;
+    const int j0 = jt * KT;
     __syncthreads();
     ck.store(k_lds);
     cv.store(v_lds);
     __syncthreads();
     const float prod_in = n_prod;
     if (jt + 1 < n_kt) {
-      const int jn = j0 + kBlockK;
+      const int jn = j0 + KT;
       ck.load(ksrc, jn);
       cv.load(vsrc, jn);
       n_prod = carry[carry_slot(jt + 1)];
     }
     // For the key-stationary kernel: C just below each 32-key sub-tile, for every row of the tile.
-    const int64_t slot_lo = carry_offset(2 * jt, n_qt) + (qi - kBlockQ * (jt >> 1));
-    const int64_t slot_hi = carry_offset(2 * jt + 1, n_qt) + (qi - kBlockQ * (jt >> 1));
+    const int u_lo = NT == 2 ? 2 * jt : jt;
+    const int64_t slot_lo = carry_offset(u_lo, n_qt) + (qi - kBlockQ * (u_lo >> 2));
+    const int64_t slot_hi = carry_offset(u_lo + 1, n_qt) + (qi - kBlockQ * (u_lo >> 2));     // NT == 2 only
     if (half == 0) prefix_out[slot_lo] = prefix;
     if (j0 > w_last - 1 + ac) {
-      if (half == 0) prefix_out[slot_hi] = prefix;
+      if (NT == 2 && half == 0) prefix_out[slot_hi] = prefix;
       continue;
     }
-    const bool diagonal = (j0 + kBlockK - 1) > (w_first - 1 + ac) || w_last >= L;
+    const bool diagonal = (j0 + KT - 1) > (w_first - 1 + ac) || w_last >= L;
 
-    f32x16 s[2], dp[2];
+    f32x16 s[NT], dp[NT];
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++) {
+    for (int mt = 0; mt < NT; mt++) {
 #pragma unroll
       for (int r = 0; r < 16; r++) { s[mt][r] = 0.f; dp[mt][r] = 0.f; }
-      const int krow = mfma_row_to_key(mt, col);
+      const int krow = NT == 2 ? mfma_row_to_key(mt, col) : mfma_row_to_key32(col);
 #pragma unroll
       for (int kk = 0; kk < kSteps; kk++) {
         vec8 a = lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half);
@@ -120,21 +126,21 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(BwdParams p) {
         dp[mt] = Elem<T>::mfma(a, dof[kk], dp[mt]);
       }
     }
-    const int lim = row_ok ? qi + ac - j0 - 32 * half : 0;
-    uint32_t pk[16], dzk[16];
+    const int lim = row_ok ? qi + ac - j0 - (KT / 2) * half : 0;
+    uint32_t pk[8 * NT], dzk[8 * NT];
     float prod_lower, prefix_upper;
-    bwd_tile_math<T, 2>(s, dp, p.scale_log2, diagonal, lim, half, drem, prod_in, prefix, pk, dzk, prod_lower,
-                        prefix_upper, prefix);
-    if (half == 0) prefix_out[slot_hi] = prefix_upper;
+    bwd_tile_math<T, NT>(s, dp, p.scale_log2, diagonal, lim, half, drem, prod_in, prefix, pk, dzk, prod_lower,
+                         prefix_upper, prefix);
+    if (NT == 2 && half == 0) prefix_out[slot_hi] = prefix_upper;
 
     // dQ += dZ K: A = dZ from registers, B = K gathered down the keys.
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
+    for (int c = 0; c < KT / 16; c++) {
       u32x4 av = {dzk[4 * c], dzk[4 * c + 1], dzk[4 * c + 2], dzk[4 * c + 3]};
       vec8 a = as_vec8<T>(av);
 #pragma unroll
       for (int dt = 0; dt < kDTiles; dt++) {
-        vec8 b = lds_col8<T>(k_lds, kRowStride, 32 * half + 8 * c, 32 * dt, lane);
+        vec8 b = lds_col8<T>(k_lds, kRowStride, (KT / 2) * half + 8 * c, 32 * dt, lane);
         dqacc[dt] = Elem<T>::mfma(a, b, dqacc[dt]);
       }
     }
@@ -156,13 +162,13 @@ template <typename T>
 static hipError_t launch_t(const BwdParams& p, int max_tiles, hipStream_t stream) {
   const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kThreads);
   if (p.vec_ok && p.head_dim == 128) {
-    hipLaunchKernelGGL((bwd_dq_kernel<T, 128, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 128, true, 32>), grid, block, 0, stream, p);
   } else if (p.vec_ok && p.head_dim == 64) {
-    hipLaunchKernelGGL((bwd_dq_kernel<T, 64, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 64, true, 64>), grid, block, 0, stream, p);
   } else if (p.head_dim <= 64) {
-    hipLaunchKernelGGL((bwd_dq_kernel<T, 64, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 64, false, 64>), grid, block, 0, stream, p);
   } else {
-    hipLaunchKernelGGL((bwd_dq_kernel<T, 128, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 128, false, 64>), grid, block, 0, stream, p);
   }
   return hipGetLastError();
 }

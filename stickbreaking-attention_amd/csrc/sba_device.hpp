@@ -75,6 +75,13 @@ __device__ __forceinline__ float fast_min(float a, float b) {
   return r;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the vector-memory counter, which
+// would stall on global loads that were deliberately left in flight across the barrier (register prefetch of
+// the next tile).  Nothing here communicates through global memory inside a kernel.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // Value held by the other half-wave (lane ^ 32).
 __device__ __forceinline__ float other_half(float x, int half) {
   uint32_t u = __builtin_bit_cast(uint32_t, x);

@@ -16,14 +16,16 @@
 
 namespace sba {
 
-template <typename T, int DH, bool kFast>
-__global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FwdParams p) {
+template <typename T, int DH, bool kFast, int KT, int kMinWaves>
+__global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
+  constexpr int NT = KT / 32;         // MFMA row tiles per key tile: a lane owns N = 16*NT consecutive keys
+  constexpr int N = 16 * NT;
   typedef typename Elem<T>::vec8 vec8;
   constexpr int kRowStride = lds_stride<DH>();
   constexpr int kSteps = DH / 16;    // MFMA k-steps over head_dim
   constexpr int kDTiles = DH / 32;   // 32-wide output tiles over head_dim
-  __shared__ __attribute__((aligned(16))) T k_lds[kBlockK * kRowStride];
-  __shared__ __attribute__((aligned(16))) T v_lds[kBlockK * kRowStride];
+  __shared__ __attribute__((aligned(16))) T k_lds[KT * kRowStride];
+  __shared__ __attribute__((aligned(16))) T v_lds[KT * kRowStride];
 
   int head, slot;
   xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
@@ -45,7 +47,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FwdParams p) {
 
   const int last_row = min(q0 + kBlockQ, L) - 1;
   const int last_key = last_row - 1 + ac;                    // last key any row of this tile can see
-  const int n_kt = last_key < 0 ? 0 : last_key / kBlockK + 1;
+  const int n_kt = last_key < 0 ? 0 : last_key / KT + 1;
   const int w_first = q0 + wave * 32, w_last = w_first + 31;   // this wave's rows
 
   f32x16 oacc[kDTiles];
@@ -58,39 +60,40 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FwdParams p) {
   float* carry = p.carry ? p.carry + (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] : nullptr;
 
   const RowSource<T> ksrc = make_row_source<T, kFast>(kb, p.k.st, L, D), vsrc = make_row_source<T, kFast>(vb, p.v.st, L, D);
-  TileCopy<T, DH, kBlockK, kFast> ck, cv;
+  TileCopy<T, DH, KT, kFast> ck, cv;
   if (n_kt > 0) {
-    ck.load(ksrc, (n_kt - 1) * kBlockK);
-    cv.load(vsrc, (n_kt - 1) * kBlockK);
+    ck.load(ksrc, (n_kt - 1) * KT);
+    cv.load(vsrc, (n_kt - 1) * KT);
   }
   for (int jt = n_kt - 1; jt >= 0; --jt) {
-    const int j0 = jt * kBlockK;
+    const int j0 = jt * KT;
     __syncthreads();
     ck.store(k_lds);
     cv.store(v_lds);
     __syncthreads();
     if (jt > 0) {
-      const int jn = j0 - kBlockK;
+      const int jn = j0 - KT;
       ck.load(ksrc, jn);
       cv.load(vsrc, jn);
     }
     // For the backward: the product over the keys between the upper 32-key sub-tile and the row, for every row
     // of the tile (the lower sub-tile's value follows once this tile's upper half is known).
-    const int64_t cslot = qi - kBlockQ * (jt >> 1);
-    if (carry && half == 0) carry[carry_offset(2 * jt + 1, n_qt) + cslot] = prod;
+    const int u_hi = NT == 2 ? 2 * jt + 1 : jt;                // sub-tile at the upper edge of this tile
+    const int64_t cslot = qi - kBlockQ * (u_hi >> 2);
+    if (carry && half == 0) carry[carry_offset(u_hi, n_qt) + cslot] = prod;
     if (j0 > w_last - 1 + ac) {                               // nothing visible to this wave yet
-      if (carry && half == 0) carry[carry_offset(2 * jt, n_qt) + cslot] = prod;
+      if (NT == 2 && carry && half == 0) carry[carry_offset(u_hi - 1, n_qt) + cslot] = prod;
       continue;
     }
-    const bool diagonal = (j0 + kBlockK - 1) > (w_first - 1 + ac);
+    const bool diagonal = (j0 + KT - 1) > (w_first - 1 + ac);
 
     // S^T tile: rows = keys (permuted so that a lane ends up with 32 consecutive keys), columns = queries.
-    f32x16 s[2];
+    f32x16 s[NT];
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++) {
+    for (int mt = 0; mt < NT; mt++) {
 #pragma unroll
       for (int r = 0; r < 16; r++) s[mt][r] = 0.f;
-      const int krow = mfma_row_to_key(mt, col);
+      const int krow = NT == 2 ? mfma_row_to_key(mt, col) : mfma_row_to_key32(col);
 #pragma unroll
       for (int kk = 0; kk < kSteps; kk++) {
         vec8 a = lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half);
@@ -98,15 +101,15 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FwdParams p) {
       }
     }
 
-    // This lane's 32 keys are j0 + 32*half + R, R = 16*mt + r, swept from R = 31 down.
+    // This lane's N keys are j0 + N*half + R, R = 16*mt + r, swept from R = N-1 down.
     //   t[R] = e[R] * prod_{R' >= R} 1/(1+e[R'])   (the weight of key R up to the product carried into the tile)
     // Hidden keys (diagonal tiles only) get e = 0: factor 1, weight 0.
-    float t[32];
+    float t[N];
     float run = 1.f;
     if (diagonal) {
-      const int lim = qi + ac - j0 - 32 * half;               // key R is visible iff R < lim
+      const int lim = qi + ac - j0 - N * half;                // key R is visible iff R < lim
 #pragma unroll
-      for (int R = 31; R >= 0; --R) {
+      for (int R = N - 1; R >= 0; --R) {
         float x = fast_min(s[R >> 4][R & 15] * p.scale_log2, kExpClamp);
         x = (R < lim) ? x : -INFINITY;
         const float e = fast_exp2(x);
@@ -115,7 +118,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FwdParams p) {
       }
     } else {
 #pragma unroll
-      for (int R = 31; R >= 0; --R) {
+      for (int R = N - 1; R >= 0; --R) {
         const float e = fast_exp2(fast_min(s[R >> 4][R & 15] * p.scale_log2, kExpClamp));
         run *= fast_rcp(1.f + e);
         t[R] = e * run;
@@ -124,19 +127,19 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FwdParams p) {
     const float oth = other_half(run, half);
     // The upper half-wave holds the higher keys, which come first in the sweep.
     const float seed = half ? prod : prod * oth;
-    if (carry && half == 0) carry[carry_offset(2 * jt, n_qt) + cslot] = seed;   // product above the lower sub-tile
+    if (NT == 2 && carry && half == 0) carry[carry_offset(u_hi - 1, n_qt) + cslot] = seed;   // product above the lower sub-tile
     prod = (prod * oth) * run;
 
     // O += P V: A = P from registers (k index <-> key 32*half + 8c + t), B = V gathered down the keys.
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
+    for (int c = 0; c < KT / 16; c++) {
       u32x4 av;
 #pragma unroll
       for (int i = 0; i < 4; i++) av[i] = pack2<T>(t[8 * c + 2 * i] * seed, t[8 * c + 2 * i + 1] * seed);
       vec8 a = as_vec8<T>(av);
 #pragma unroll
       for (int dt = 0; dt < kDTiles; dt++) {
-        vec8 b = lds_col8<T>(v_lds, kRowStride, 32 * half + 8 * c, 32 * dt, lane);
+        vec8 b = lds_col8<T>(v_lds, kRowStride, N * half + 8 * c, 32 * dt, lane);
         oacc[dt] = Elem<T>::mfma(a, b, oacc[dt]);
       }
     }
@@ -164,13 +167,13 @@ template <typename T>
 static hipError_t launch_fwd_t(const FwdParams& p, int max_tiles, hipStream_t stream) {
   const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kThreads);
   if (p.vec_ok && p.head_dim == 128) {
-    hipLaunchKernelGGL((fwd_kernel<T, 128, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<T, 128, true, 32, 3>), grid, block, 0, stream, p);
   } else if (p.vec_ok && p.head_dim == 64) {
-    hipLaunchKernelGGL((fwd_kernel<T, 64, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<T, 64, true, 64, 2>), grid, block, 0, stream, p);
   } else if (p.head_dim <= 64) {
-    hipLaunchKernelGGL((fwd_kernel<T, 64, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<T, 64, false, 64, 2>), grid, block, 0, stream, p);
   } else {
-    hipLaunchKernelGGL((fwd_kernel<T, 128, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<T, 128, false, 64, 2>), grid, block, 0, stream, p);
   }
   return hipGetLastError();
 }
