@@ -189,8 +189,8 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
 // One workgroup = 8 waves = one 64-key tile, swept by query tiles of 64 rows.  Waves 0-3 are PRODUCERS: wave
 // (rg, g) takes rows 32*rg .. +31 against the 32-key sub-tile g (one MFMA row tile, 16 keys per lane, that
 // sub-tile's K/V operands stationary in registers), recomputes P^T and dZ^T and writes them to LDS.  Waves 4-7
-// are CONSUMERS: one step behind, wave cw contracts P^T/dZ^T with dO/Q over the 64 rows into the
-// 64-key x 32-column block cw of dV and dK.  Every SIMD hosts one producer (exp/rcp/VALU bound) and one consumer
+// are CONSUMERS: they stage the query tiles (Q, dO) into LDS and, one step behind, wave cw contracts P^T/dZ^T
+// with dO/Q over the 64 rows into the 64-key x 32-column block cw of dV and dK.  Every SIMD hosts one producer (exp/rcp/VALU bound) and one consumer
 // (MFMA/LDS bound), so the two pipelines overlap, and there is ONE barrier per step: P/dZ are double-buffered
 // and Q/dO triple-buffered (written for step t+1, read by producers for step t and by consumers for step t-1).
 // The per-(row, sub-tile) carries are what the forward and the dQ kernel recorded at 32-key granularity.
@@ -255,10 +255,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
         vf[kk] = as_vec8<T>(load_row8<T, true>(vb + (int64_t)key * p.v.st, 16 * kk + 8 * half, D, key < L));
       }
     }
-    const RowSource<T> qsrc = make_row_source<T, true>(qb, p.q.st, L, D), dosrc = make_row_source<T, true>(dob, p.d_o.st, L, D);
-    // Per-row scalars (drem, product above the sub-tile, C below it) are fetched one step ahead and BEFORE the
-    // tile prefetch of that step: memory results return in order, so a scalar consumed right after a younger
-    // tile load was issued would drain the whole prefetch.
+    // Per-row scalars (drem, product above the sub-tile, C below it), fetched one step ahead.
     T n_drem = (T)0.f;
     float n_prod = 1.f, n_prefix = 0.f;
     auto fetch_row_scalars = [&](int row0) {
@@ -267,19 +264,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
       n_prod = carry[r];
       n_prefix = prefix[r];
     };
-    TileCopy<T, DH, kDkvRows, true> cq, cdo;
-    if (n_steps > 0) {
-      fetch_row_scalars(row_begin);
-      cq.load(qsrc, row_begin);
-      cdo.load(dosrc, row_begin);
-      cq.store(lds + Lds::kQ);
-      cdo.store(lds + Lds::kQ + Lds::kQdoTile);
-      if (n_steps > 1) {
-        const int qn = row_begin + kDkvRows;
-        cq.load(qsrc, qn);
-        cdo.load(dosrc, qn);
-      }
-    }
+    if (n_steps > 0) fetch_row_scalars(row_begin);
     __syncthreads();
     for (int t = 0; t <= n_steps; ++t) {
       if (t < n_steps) {
@@ -288,20 +273,8 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
         const T* do_lds = q_lds + Lds::kQdoTile;
         T* p_lds = lds + Lds::kP + (t & 1) * 2 * Lds::kPTile;
         T* dz_lds = p_lds + Lds::kPTile;
-        // Stage the next query tile (fetched during the previous step) and start fetching the one after; the
-        // barrier that ends this step is the only point that waits for these loads.
         const float drem = (float)n_drem, prod_in = n_prod, prefix_in = n_prefix;
         if (t + 1 < n_steps) fetch_row_scalars(q0 + kDkvRows);
-        if (t + 1 < n_steps) {
-          T* nq_lds = lds + Lds::kQ + ((t + 1) % 3) * 2 * Lds::kQdoTile;
-          cq.store(nq_lds);
-          cdo.store(nq_lds + Lds::kQdoTile);
-          if (t + 2 < n_steps) {
-            const int qn = q0 + 2 * kDkvRows;
-            cq.load(qsrc, qn);
-            cdo.load(dosrc, qn);
-          }
-        }
         const int w_first = q0 + rg * 32, w_last = w_first + 31;
         const int qi = w_first + col;
         const bool row_ok = qi < L;
@@ -351,8 +324,35 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
     for (int b = 0; b < 2; b++)
 #pragma unroll
       for (int r = 0; r < 16; r++) { dkacc[b][r] = 0.f; dvacc[b][r] = 0.f; }
+    // The consumers also move the query tiles global -> registers -> LDS (they have the issue slots to spare):
+    // tile t+1 is written at the top of step t from registers loaded during step t-1, then tile t+2 is requested;
+    // the barrier that ends a step is the only point that waits for those loads.
+    const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
+    const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
+    const RowSource<T> qsrc = make_row_source<T, true>(qb, p.q.st, L, D), dosrc = make_row_source<T, true>(dob, p.d_o.st, L, D);
+    TileCopy<T, DH, kDkvRows, true> cq, cdo;
+    if (n_steps > 0) {
+      cq.load(qsrc, row_begin);
+      cdo.load(dosrc, row_begin);
+      cq.store(lds + Lds::kQ);
+      cdo.store(lds + Lds::kQ + Lds::kQdoTile);
+      if (n_steps > 1) {
+        cq.load(qsrc, row_begin + kDkvRows);
+        cdo.load(dosrc, row_begin + kDkvRows);
+      }
+    }
     __syncthreads();
     for (int t = 0; t <= n_steps; ++t) {
+      if (t + 1 < n_steps) {
+        T* nq_lds = lds + Lds::kQ + ((t + 1) % 3) * 2 * Lds::kQdoTile;
+        cq.store(nq_lds);
+        cdo.store(nq_lds + Lds::kQdoTile);
+        if (t + 2 < n_steps) {
+          const int qn = row_begin + (t + 2) * kDkvRows;
+          cq.load(qsrc, qn);
+          cdo.load(dosrc, qn);
+        }
+      }
       if (t >= 1) {
         const int u = t - 1;
         const T* q_lds = lds + Lds::kQ + (u % 3) * 2 * Lds::kQdoTile;
