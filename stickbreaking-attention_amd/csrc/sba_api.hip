@@ -10,7 +10,7 @@ hipError_t launch_fwd(const FwdParams& p, int dtype_is_f16, int max_tiles, hipSt
 hipError_t launch_bwd_dq(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
 hipError_t launch_bwd_dkv(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
 hipError_t launch_fwd_f32(const FwdParams& p, int max_tiles, hipStream_t stream);
-hipError_t launch_bwd_f32(const BwdParams& p, int max_q_tiles, int max_k_tiles, hipStream_t stream);
+hipError_t launch_bwd_f32(const BwdParams& p, int batches, int64_t tokens, int max_q_tiles, hipStream_t stream);
 }  // namespace sba
 
 namespace {
@@ -220,7 +220,7 @@ int sba_bwd(const SbaArgs* a) {
   hipEvent_t* ev = (hipEvent_t*)a->trace_events;
   if (ev && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;
   if (a->dtype == SBA_F32) {
-    if (sba::launch_bwd_f32(p, (int)L.max_q_tiles, (int)L.max_k_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
+    if (sba::launch_bwd_f32(p, fixed ? a->num_seqs : 1, a->total_tokens, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
     if (ev && (hipEventRecord(ev[1], stream) != hipSuccess || hipEventRecord(ev[2], stream) != hipSuccess)) return SBA_ERR_LAUNCH;
     return SBA_OK;
   }

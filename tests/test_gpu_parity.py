@@ -100,6 +100,43 @@ def test_small_f16(gpu_device):
         tol_check(n, a, b, torch.float16, "f16")
 
 
+def test_config1_fp32(gpu_device):
+    # The reference's CPU-runnable configuration: fp32, H=4, D=64, lengths [128, 256, 64], seed 0, zero_start=False.
+    # Checked against the DENSE restatement of sb_ref.py (per-sequence calls, gradients by autograd) in fp32 and
+    # against the fp64 streaming form; bar 1e-4 on o, rem, dq, dk, dv.
+    inp = bench.make_inputs("c1", gpu_device)
+    host = [inp[n].cpu() for n in ("q", "k", "v", "do", "drem")]
+    cu = inp["cu"].cpu()
+    dense = orc.dense_backward_autograd(host[0], host[1], host[2], cu, host[3], host[4])
+    ref64 = orc.varlen_stream(host[0], host[1], host[2], cu, do=host[3], drem=host[4], dtype=torch.float64)
+    got = run_varlen(inp["q"], inp["k"], inp["v"], inp["cu"], inp["lengths"], False, False, inp["do"], inp["drem"])
+    for n, a, b, c in zip(NAMES, got, dense, ref64):
+        tol_check(n, a, b, torch.float32, "c1 vs dense fp32")
+        tol_check(n, a, c, torch.float32, "c1 vs fp64")
+
+
+@pytest.mark.parametrize("attend_current", [False, True])
+def test_fp32_ragged_and_fixed(gpu_device, attend_current):
+    from stickbreaking_attention import sb_attn
+
+    lengths = [1, 5, 64, 65, 129, 300]
+    host, dev, cu = small_case(2, 128, lengths, torch.float32, seed=11)
+    ref = orc.varlen_stream(*host[:3], cu, attend_current=attend_current, do=host[3], drem=host[4], dtype=torch.float64)
+    got = run_varlen(*dev[:3], cu.to(gpu_device), lengths, False, attend_current, dev[3], dev[4])
+    for n, a, b in zip(NAMES, got, ref):
+        tol_check(n, a, b, torch.float32, "f32 ragged")
+    B, H, L, D = 2, 3, 200, 50
+    g = torch.Generator().manual_seed(12)
+    q, k, v, do = (torch.randn(B, H, L, D, generator=g) for _ in range(4))
+    drem = torch.randn(B, H, L, generator=g)
+    ref = orc.fixed_stream(q, k, v, attend_current=attend_current, do=do, drem=drem, dtype=torch.float64)
+    qd, kd, vd = (t.to(gpu_device).requires_grad_() for t in (q, k, v))
+    o, rem = sb_attn(qd, kd, vd, attend_current=attend_current)
+    grads = torch.autograd.grad([o, rem], [qd, kd, vd], [do.to(gpu_device), drem.to(gpu_device)])
+    for n, a, b in zip(NAMES, [o, rem, *grads], ref):
+        tol_check(n, a, b, torch.float32, "f32 fixed")
+
+
 def test_zero_start_forms_and_int64_cu_agree(gpu_device):
     lengths = [77, 300, 1, 64]
     host, dev, cu = small_case(4, 64, lengths, torch.bfloat16, seed=3)
