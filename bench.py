@@ -28,6 +28,12 @@ sys.path.insert(0, os.path.join(ROOT, "stickbreaking-attention_amd"))
 
 MFMA_BF16_PEAK = 2.5e15          # MI355X dense bf16 MFMA peak, FLOP/s
 
+# HBM bytes per launch (fetch + write) of each kernel on workload c3, from `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` runs of `bench.py --traffic-probe`, each scaled by what the same counter read for the probe's
+# 1 GiB device-to-device copy.  Hardware counters cannot be read from inside this script, so the figures are carried
+# here; they are reported only for the workload they were measured on.
+MEASURED_TRAFFIC_BYTES = {"c3": {"fwd_kernel": 1.955e9, "bwd_dq_kernel": 1.958e9, "bwd_dkv_kernel": 2.556e9}}
+
 
 # ----------------------------------------------------------------------------------------------
 # Synthetic workloads (the five configurations the baseline names); shared with the tests.
@@ -143,24 +149,27 @@ def time_kernels(inp, native, iters):
     return [s / iters for s in sums]
 
 
-def cpu_baseline(sample_len=1536):
-    """Dense fp32 restatement of the reference algorithm (oracle/, a port) on the host: forward + backward of ONE
-    (head, sequence) slice, head_dim 128, through autograd as the reference's tests obtain gradients."""
+def cpu_baseline(sample_len=4096, budget_s=15.0):
+    """The CPU restatement (dense fp32 forward + autograd backward) timed on (head, sequence) slices of the bench
+    workload's shape, one after another until about `budget_s` seconds of CPU work have been spent."""
     sys.path.insert(0, ROOT)
     from oracle import sb_oracle as orc
 
     D = 128
     g = torch.Generator().manual_seed(0)
-    q, k, v, do = (torch.randn(1, sample_len, D, generator=g) for _ in range(4))
-    drem = torch.randn(1, sample_len, generator=g)
     threads = torch.get_num_threads()
-    t0 = time.perf_counter()
-    orc.dense_backward_autograd(q, k, v, [sample_len], do, drem)
-    dt = time.perf_counter() - t0
-    flops = 14 * D * visible_pairs([sample_len], 1)
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"fwd+bwd of one (head, sequence) slice, L={sample_len}, D=128, fp32 dense O(L^3) restatement "
-                      f"of sb_ref.py via autograd, {dt:.2f} s, os.cpu_count()={os.cpu_count()}"}
+    slices, spent = 0, 0.0
+    while spent < budget_s:
+        q, k, v, do = (torch.randn(1, sample_len, D, generator=g) for _ in range(4))
+        drem = torch.randn(1, sample_len, generator=g)
+        t0 = time.perf_counter()
+        orc.dense_backward_autograd(q, k, v, [sample_len], do, drem)
+        spent += time.perf_counter() - t0
+        slices += 1
+    flops = 14 * D * visible_pairs([sample_len], 1) * slices
+    return {"value": flops / spent / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"fwd+bwd of {slices} (head, sequence) slices, L={sample_len}, D=128, fp32 dense restatement of "
+                      f"sb_ref.py via autograd, {spent:.1f} s, os.cpu_count()={os.cpu_count()}"}
 
 
 def main():
@@ -170,6 +179,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also launch one plain 1 GiB device copy, the known-size reference for HBM traffic counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (the operator shards by head or by sequence with no "
@@ -204,6 +215,13 @@ def main():
                 sb_attn(*(t.view(H, B, L, D).transpose(0, 1) for t in (q, k, v)))
             else:
                 sb_attn_varlen(q, k, v, inp["cu"], max(lengths), zero_start=inp["zero_start"])
+
+    if args.traffic_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -249,7 +267,8 @@ def main():
                 "frac_bf16_mfma_peak": 4 * D * pairs / (ms_fwd * 1e-3) / MFMA_BF16_PEAK},
         "kernels_ms": {n: round(kernels[n][0], 4) for n in kernels},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": MFMA_BF16_PEAK / 1e12, "unit": "TFLOP/s",
-                     "frac": achieved * 1e12 / MFMA_BF16_PEAK, "traffic": None},
+                     "frac": achieved * 1e12 / MFMA_BF16_PEAK,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dom)},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
