@@ -11,6 +11,8 @@ from typing import Optional
 
 import torch
 
+from .utils import custom_op
+
 _LIB_NAME = "libsba.so"
 _lib = None
 # Optional ctypes array of hipEvent_t handed to the next calls as SbaArgs.trace_events (benchmarks only).
@@ -140,45 +142,43 @@ def prepare_cu_seqlens(cu_seqlens: torch.Tensor, device) -> torch.Tensor:
     return cu_seqlens.contiguous()
 
 
-def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, want_carry):
-    """Launch the forward.  Returns (o, rem, row_stat, carry or None).  Packed mode when cu_seqlens is given.
-    ``carry`` is the buffer the backward needs; it is only produced when ``want_carry``."""
-    _require_gpu(q, k, v)
+def carry_elems(num_heads: int, total_tokens: int, num_seqs: int, max_seqlen, fixed: bool) -> int:
+    """fp32 elements of the ``carry`` buffer the forward fills for the backward: the same bound the library
+    reports through ``sba_workspace_bytes`` (one value per query row and 32-key sub-tile the row sweeps),
+    computed here from shapes alone so that it can be traced by torch.compile."""
+    T, B = total_tokens, num_seqs
+    if fixed:
+        m = -(-T // 128)
+        slots = B * 256 * m * (m + 1)
+    else:
+        max_len = max_seqlen if (max_seqlen and 0 < max_seqlen < T) else T
+        slots = -(-(T * max_len) // 64) + 6 * T + 512 * B
+    nbytes = -(-(slots * num_heads * 4) // 256) * 256
+    return nbytes // 4
+
+
+def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, o, rem, neg_log_acc, carry):
     fixed = cu_seqlens is None
-    q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)
     with torch.cuda.device(q.device):
         a = _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current)
-        o = torch.empty_like(q)
-        if o.stride(-1) != 1:
-            o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-        rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
-        row_stat = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
         a.q, a.k, a.v, a.o = (_tensor(t, fixed) for t in (q, k, v, o))
         a.rem = _vector(rem, fixed)
-        a.row_stat = row_stat.data_ptr()
+        a.row_stat = neg_log_acc.data_ptr()
         need, need_carry = ctypes.c_size_t(0), ctypes.c_size_t(0)
         _check(lib().sba_workspace_bytes(ctypes.byref(a), ctypes.byref(need), None, ctypes.byref(need_carry)), "sba_workspace_bytes")
         ws = torch.empty(need.value, dtype=torch.uint8, device=q.device)
         a.workspace, a.workspace_bytes = ws.data_ptr(), need.value
-        carry = None
-        if want_carry:
-            carry = torch.empty(need_carry.value // 4, dtype=torch.float32, device=q.device)
+        if carry.numel() > 0:
+            if carry.numel() * 4 < need_carry.value:
+                raise RuntimeError(f"carry buffer too small: {carry.numel() * 4} < {need_carry.value} bytes")
             a.carry = carry.data_ptr()
         _check(lib().sba_fwd(ctypes.byref(a)), "sba_fwd")
-    return o, rem, row_stat, carry
 
 
-def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current):
-    """Launch the backward.  Returns (dq, dk, dv)."""
-    _require_gpu(q, k, v, do, drem, carry)
+def _launch_bwd(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, dq, dk, dv):
     fixed = cu_seqlens is None
-    do = rows_contiguous(do)
-    q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)
     with torch.cuda.device(q.device):
         a = _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current)
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-        if drem is not None and drem.dtype != q.dtype:
-            drem = drem.to(q.dtype)
         a.q, a.k, a.v, a.d_o, a.dq, a.dk, a.dv = (_tensor(t, fixed) for t in (q, k, v, do, dq, dk, dv))
         a.d_rem = _vector(drem, fixed)
         a.carry = carry.data_ptr()
@@ -187,4 +187,80 @@ def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seql
         ws = torch.empty(need.value, dtype=torch.uint8, device=q.device)
         a.workspace, a.workspace_bytes = ws.data_ptr(), need.value
         _check(lib().sba_bwd(ctypes.byref(a)), "sba_bwd")
+
+
+# The four launchers as out-parameter operators, registered for torch.compile the way the reference registers
+# its own (sb_varlen_fwd.py:453, sb_varlen_bwd.py:541, sb_attn/sb_fwd.py:175, sb_attn/sb_bwd.py:207).  ``carry``
+# replaces the reference's use of the saved ``neg_log_acc`` in the backward; an empty ``carry`` means "forward
+# only".
+@custom_op("varlen_fwd", mutates_args={"o", "rem", "neg_log_acc", "carry"})
+def varlen_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor, cu_has_leading_zero: bool,
+               max_seqlens: int, logit_scale: float, attend_current: bool, o: torch.Tensor, rem: torch.Tensor,
+               neg_log_acc: torch.Tensor, carry: torch.Tensor) -> None:
+    _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlens, logit_scale, attend_current, o, rem, neg_log_acc, carry)
+
+
+@custom_op("varlen_bwd", mutates_args={"dq", "dk", "dv"})
+def varlen_bwd(do: torch.Tensor, drem: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, carry: torch.Tensor,
+               cu_seqlens: torch.Tensor, cu_has_leading_zero: bool, max_seqlens: int, logit_scale: float,
+               attend_current: bool, dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor) -> None:
+    _launch_bwd(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlens, logit_scale, attend_current, dq, dk, dv)
+
+
+@custom_op("attn_fwd", mutates_args={"o", "rem", "neg_log_acc", "carry"})
+def attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_scale: float, attend_current: bool,
+             o: torch.Tensor, rem: torch.Tensor, neg_log_acc: torch.Tensor, carry: torch.Tensor) -> None:
+    _launch_fwd(q, k, v, None, False, q.size(2), logit_scale, attend_current, o, rem, neg_log_acc, carry)
+
+
+@custom_op("attn_bwd", mutates_args={"dq", "dk", "dv"})
+def attn_bwd(do: torch.Tensor, drem: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, carry: torch.Tensor,
+             logit_scale: float, attend_current: bool, dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor) -> None:
+    _launch_bwd(do, drem, q, k, v, carry, None, False, q.size(2), logit_scale, attend_current, dq, dk, dv)
+
+
+def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, want_carry):
+    """Launch the forward.  Returns (o, rem, row_stat, carry or None).  Packed mode when cu_seqlens is given.
+    ``carry`` is the buffer the backward needs; it is only produced when ``want_carry``."""
+    _require_gpu(q, k, v)
+    fixed = cu_seqlens is None
+    q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)
+    if q.dtype not in _DTYPES:
+        raise TypeError(f"unsupported dtype {q.dtype}")
+    o = torch.empty_like(q)
+    if o.stride(-1) != 1:
+        o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
+    row_stat = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
+    n_carry = 0
+    if want_carry:
+        if fixed:
+            n_carry = carry_elems(q.size(1), q.size(2), q.size(0), None, True)
+        else:
+            n_carry = carry_elems(q.size(0), q.size(1), cu_seqlens.numel() - (1 if cu_has_leading_zero else 0), max_seqlen, False)
+    carry = torch.empty(n_carry, dtype=torch.float32, device=q.device)
+    if fixed:
+        attn_fwd(q, k, v, float(logit_scale), bool(attend_current), o, rem, row_stat, carry)
+    else:
+        varlen_fwd(q, k, v, cu_seqlens, bool(cu_has_leading_zero), int(max_seqlen) if max_seqlen else 0, float(logit_scale),
+                   bool(attend_current), o, rem, row_stat, carry)
+    return o, rem, row_stat, (carry if want_carry else None)
+
+
+def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current):
+    """Launch the backward.  Returns (dq, dk, dv)."""
+    _require_gpu(q, k, v, do, drem, carry)
+    fixed = cu_seqlens is None
+    do = rows_contiguous(do)
+    q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if drem is None:
+        drem = torch.zeros(q.shape[:-1], dtype=q.dtype, device=q.device)
+    elif drem.dtype != q.dtype:
+        drem = drem.to(q.dtype)
+    if fixed:
+        attn_bwd(do, drem, q, k, v, carry, float(logit_scale), bool(attend_current), dq, dk, dv)
+    else:
+        varlen_bwd(do, drem, q, k, v, carry, cu_seqlens, bool(cu_has_leading_zero), int(max_seqlen) if max_seqlen else 0,
+                   float(logit_scale), bool(attend_current), dq, dk, dv)
     return dq, dk, dv

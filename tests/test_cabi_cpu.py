@@ -84,6 +84,37 @@ def test_workspace_sizes_cover_any_batch(native):
     assert carry.value == -(-(4 * 256 * 4 * 5 * 3 * 4) // 256) * 256
 
 
+def test_python_carry_size_matches_library(native):
+    """The operators size the carry buffer from shapes alone (traceable by torch.compile); that formula must
+    agree with what the library reports."""
+    lib = native.lib()
+    rng = np.random.default_rng(1)
+    carry = ctypes.c_size_t()
+    for _ in range(200):
+        H, B, T = int(rng.integers(1, 40)), int(rng.integers(1, 50)), int(rng.integers(1, 100000))
+        for hint in (0, int(rng.integers(1, T + 1)), T + 5):
+            a = _args(native, H, 64, T, B, max_seqlen=hint)
+            assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, ctypes.byref(carry)) == 0
+            assert native.carry_elems(H, T, B, hint, False) * 4 == carry.value
+        a = _args(native, H, 64, T, B, varlen=False)
+        assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, ctypes.byref(carry)) == 0
+        assert native.carry_elems(H, T, B, None, True) * 4 == carry.value
+
+
+def test_custom_ops_are_registered(native):
+    """The four launchers are torch.library operators named like the reference's (utils.py:20-40 with
+    sb_varlen_fwd.py:453, sb_varlen_bwd.py:541, sb_attn/sb_fwd.py:175, sb_attn/sb_bwd.py:207), out-parameter style."""
+    from stickbreaking_attention import utils
+
+    assert utils.PACKAGE_NAME == "stickbreaking_attention" and abs(utils.inv_log2 - 1.4426950408889634) < 1e-15
+    ns = torch.ops.stickbreaking_attention
+    for name, mutated in (("varlen_fwd", ("o", "rem", "neg_log_acc", "carry")), ("varlen_bwd", ("dq", "dk", "dv")),
+                          ("attn_fwd", ("o", "rem", "neg_log_acc", "carry")), ("attn_bwd", ("dq", "dk", "dv"))):
+        schema = getattr(ns, name).default._schema
+        assert len(schema.returns) == 0
+        assert tuple(a.name for a in schema.arguments if a.alias_info is not None and a.alias_info.is_write) == mutated
+
+
 def test_size_query_validates(native):
     lib = native.lib()
     assert lib.sba_workspace_bytes(None, None, None, None) == -1

@@ -326,6 +326,39 @@ def test_forward_without_grad_skips_carry(gpu_device):
     torch.testing.assert_close(torch.exp2(stat), rem.float(), atol=4e-3, rtol=4e-3)   # row_stat = log2(rem)
 
 
+def test_torch_compile_graph_matches_eager(gpu_device):
+    """Under torch.compile the launchers run as the registered stickbreaking_attention::* operators; outputs and
+    gradients must be bit-identical to the eager call.  (aot_eager backend: graph capture and functionalisation
+    of the mutating operators without code generation.)"""
+    from stickbreaking_attention import sb_attn, sb_attn_varlen
+
+    lengths = [200, 1, 77, 130]
+    host, dev, cu = small_case(2, 128, lengths, torch.bfloat16, seed=21)
+    cu = cu.to(gpu_device)
+
+    def varlen_fn(q, k, v, do, drem):
+        o, rem = sb_attn_varlen(q, k, v, cu, max(lengths), zero_start=False)
+        return ((o.float() * do.float()).sum() + (rem.float() * drem.float()).sum()), o, rem
+
+    def fixed_fn(q, k, v, do, drem):
+        o, rem = sb_attn(q, k, v)
+        return ((o.float() * do.float()).sum() + (rem.float() * drem.float()).sum()), o, rem
+
+    for fn, shape in ((varlen_fn, None), (fixed_fn, (2, 2, 102, 128))):
+        ins = [t if shape is None or t.dim() < 3 else t[:, :204].reshape(shape) for t in dev]
+        if shape is not None:
+            ins[4] = dev[4][:, :204].reshape(shape[:-1])
+        results = []
+        for f in (fn, torch.compile(fn, backend="aot_eager")):
+            q, k, v = (t.detach().clone().requires_grad_() for t in ins[:3])
+            loss, o, rem = f(q, k, v, ins[3], ins[4])
+            loss.backward()
+            torch.cuda.synchronize()
+            results.append((o.detach(), rem.detach(), q.grad, k.grad, v.grad))
+        for name, a, b in zip(NAMES, *results):
+            assert torch.equal(a, b), f"compiled {name} differs from eager"
+
+
 def test_c_abi_rejects_bad_arguments(gpu_device):
     import ctypes
 
