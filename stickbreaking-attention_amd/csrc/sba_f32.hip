@@ -2,8 +2,8 @@
 //
 // This is the correctness path behind the 1e-4 tolerance, not a tuned one: one wave walks one query row at a
 // time, 64 keys per step with one key per lane, so the stick-breaking product and the prefix sum along the keys
-// are wave-level scans.  Workgroup = 4 waves = one 128-row query tile from the scheduler's list; wave w owns
-// rows 32w .. 32w+31.
+// are wave-level scans.  Workgroup = 4 waves = 16 consecutive rows of a 128-row query tile from the scheduler's
+// list (eight workgroups per tile, so that small problems still spread over the chip); wave w owns 4 of them.
 //
 //   forward : keys swept in reverse from the diagonal (as sb_varlen_fwd.py:155-165), running product per row;
 //             records the product above every 64-key step in `carry` (slot of the step's upper 32-key sub-tile).
@@ -19,6 +19,9 @@ namespace sba {
 
 constexpr int kF32Keys = 64;          // keys per step (one per lane)
 constexpr int kMaxD = 128;
+constexpr int kF32Rows = 16;          // query rows per workgroup
+constexpr int kF32Split = kBlockQ / kF32Rows;
+constexpr int kF32RowsPerWave = kF32Rows / kWaves;
 
 __device__ __forceinline__ float wave_bcast(float x, int lane) { return __shfl(x, lane); }
 
@@ -52,10 +55,11 @@ __device__ __forceinline__ float dot_row(const float* q_lds, const float* krow, 
 __global__ __launch_bounds__(kThreads) void fwd_f32_kernel(FwdParams p) {
   __shared__ float q_lds[kWaves][kMaxD];
   int head, slot;
-  xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
+  xcd_head_tile(blockIdx.x / kF32Split, p.num_heads, &head, &slot);
   if (slot >= p.counts[0]) return;
   const Tile tile = p.tiles[slot];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int row_base = tile.origin + (blockIdx.x % kF32Split) * kF32Rows + wave * kF32RowsPerWave;
   const int L = tile.seq_len, ac = p.attend_current, D = p.head_dim;
   const int64_t tok0 = tile.seq_start;
   const float* qb = (const float*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
@@ -65,8 +69,8 @@ __global__ __launch_bounds__(kThreads) void fwd_f32_kernel(FwdParams p) {
   const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
   float* carry = p.carry ? p.carry + (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] : nullptr;
 
-  for (int r = 0; r < 32; r++) {
-    const int i = tile.origin + wave * 32 + r;
+  for (int r = 0; r < kF32RowsPerWave; r++) {
+    const int i = row_base + r;
     if (i >= L) break;                                       // wave-uniform
     for (int d = lane; d < D; d += 64) q_lds[wave][d] = qb[(int64_t)i * p.q.st + d];
     const int last_key = i - 1 + ac;
@@ -119,17 +123,18 @@ struct BwdF32Lds {
   float d_o[kWaves][kMaxD];
   float dk[kF32Keys][kMaxD];
   float dv[kF32Keys][kMaxD];
-  float dq[kBlockQ][kMaxD];
+  float dq[kF32Rows][kMaxD];
 };
 
 __global__ __launch_bounds__(kThreads) void bwd_f32_kernel(BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   BwdF32Lds& lds = *reinterpret_cast<BwdF32Lds*>(lds_raw);
   int head, slot;
-  xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
+  xcd_head_tile(blockIdx.x / kF32Split, p.num_heads, &head, &slot);
   if (slot >= p.counts[0]) return;
   const Tile tile = p.q_tiles[slot];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wg_row0 = tile.origin + (blockIdx.x % kF32Split) * kF32Rows;      // first row of this workgroup
   const int L = tile.seq_len, ac = p.attend_current, D = p.head_dim;
   const int64_t tok0 = tile.seq_start;
   const float* qb = (const float*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
@@ -142,17 +147,17 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_kernel(BwdParams p) {
   const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
   const float* carry = p.carry + (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id];
 
-  const int tile_last_key = min(tile.origin + kBlockQ, L) - 2 + ac;
-  const int n_steps = tile_last_key < 0 ? 0 : tile_last_key / kF32Keys + 1;
-  for (int idx = threadIdx.x; idx < kBlockQ * kMaxD; idx += kThreads) (&lds.dq[0][0])[idx] = 0.f;
-  float prefix_row = 0.f;      // lane r (< 32) holds the running prefix sum C of this wave's row r
+  const int wg_last_key = min(wg_row0 + kF32Rows, L) - 2 + ac;
+  const int n_steps = (wg_last_key < 0 || wg_row0 >= L) ? 0 : wg_last_key / kF32Keys + 1;
+  for (int idx = threadIdx.x; idx < kF32Rows * kMaxD; idx += kThreads) (&lds.dq[0][0])[idx] = 0.f;
+  float prefix_row = 0.f;      // lane r (< rows per wave) holds the running prefix sum C of this wave's row r
 
   for (int c = 0; c < n_steps; ++c) {
     const int j0 = c * kF32Keys;
     for (int idx = threadIdx.x; idx < kF32Keys * kMaxD; idx += kThreads) { (&lds.dk[0][0])[idx] = 0.f; (&lds.dv[0][0])[idx] = 0.f; }
     __syncthreads();
-    for (int r = 0; r < 32; r++) {
-      const int i = tile.origin + wave * 32 + r;
+    for (int r = 0; r < kF32RowsPerWave; r++) {
+      const int i = wg_row0 + wave * kF32RowsPerWave + r;
       const int last_key = i - 1 + ac;
       if (i >= L || j0 > last_key) continue;                  // wave-uniform
       for (int d = lane; d < D; d += 64) {
@@ -192,8 +197,8 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_kernel(BwdParams p) {
           atomicAdd(&lds.dv[t][lane + 64], at * lds.d_o[wave][lane + 64]);
         }
       }
-      lds.dq[wave * 32 + r][lane] += dq0;                     // this wave is the only writer of its rows
-      lds.dq[wave * 32 + r][lane + 64] += dq1;
+      lds.dq[wave * kF32RowsPerWave + r][lane] += dq0;        // this wave is the only writer of its rows
+      lds.dq[wave * kF32RowsPerWave + r][lane + 64] += dq1;
     }
     __syncthreads();
     for (int idx = threadIdx.x; idx < kF32Keys * D; idx += kThreads) {
@@ -206,14 +211,14 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_kernel(BwdParams p) {
     __syncthreads();
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < kBlockQ * D; idx += kThreads) {
-    const int r = idx / D, d = idx % D, i = tile.origin + r;
+  for (int idx = threadIdx.x; idx < kF32Rows * D; idx += kThreads) {
+    const int r = idx / D, d = idx % D, i = wg_row0 + r;
     if (i < L) dqb[(int64_t)i * p.dq.st + d] = lds.dq[r][d] * p.logit_scale;
   }
 }
 
 hipError_t launch_fwd_f32(const FwdParams& p, int max_tiles, hipStream_t stream) {
-  hipLaunchKernelGGL(fwd_f32_kernel, dim3((unsigned)(max_tiles * p.num_heads)), dim3(kThreads), 0, stream, p);
+  hipLaunchKernelGGL(fwd_f32_kernel, dim3((unsigned)(max_tiles * p.num_heads * kF32Split)), dim3(kThreads), 0, stream, p);
   return hipGetLastError();
 }
 
@@ -224,7 +229,7 @@ hipError_t launch_bwd_f32(const BwdParams& p, int batches, int64_t tokens, int m
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_f32_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(BwdF32Lds));
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(bwd_f32_kernel, dim3((unsigned)(max_q_tiles * p.num_heads)), dim3(kThreads), sizeof(BwdF32Lds), stream, p);
+  hipLaunchKernelGGL(bwd_f32_kernel, dim3((unsigned)(max_q_tiles * p.num_heads * kF32Split)), dim3(kThreads), sizeof(BwdF32Lds), stream, p);
   return hipGetLastError();
 }
 
