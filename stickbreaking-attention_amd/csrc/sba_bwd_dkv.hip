@@ -206,9 +206,8 @@ template <int DH> struct Dkv3Lds {
   static constexpr int kElems = kP + 4 * kPTile;
 };
 
-template <typename T>
+template <typename T, int DH>
 __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
-  constexpr int DH = 128;
   typedef typename Elem<T>::vec8 vec8;
   typedef Dkv3Lds<DH> Lds;
   constexpr int kRowStride = Lds::kRowStride, kPStride = Lds::kPStride;
@@ -318,10 +317,13 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
       __syncthreads();
     }
   } else {
-    // Output blocks of this consumer wave: both 32-key row tiles x head_dim columns 32*wave .. +31.
-    f32x16 dkacc[2], dvacc[2];
+    // Output blocks of this consumer wave.  head_dim 128: both 32-key row tiles x columns 32*wave .. +31;
+    // head_dim 64: row tile wave/2 x columns 32*(wave%2) .. +31.
+    constexpr int kMT = DH == 128 ? 2 : 1;
+    const int mt0 = DH == 128 ? 0 : wave >> 1, ct = DH == 128 ? wave : wave & 1;
+    f32x16 dkacc[kMT], dvacc[kMT];
 #pragma unroll
-    for (int b = 0; b < 2; b++)
+    for (int b = 0; b < kMT; b++)
 #pragma unroll
       for (int r = 0; r < 16; r++) { dkacc[b][r] = 0.f; dvacc[b][r] = 0.f; }
     // The consumers also move the query tiles global -> registers -> LDS (they have the issue slots to spare):
@@ -363,28 +365,28 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
 #pragma unroll
         for (int c = 0; c < kDkvRows / 16; c++) {
           const int row0 = 16 * c + 8 * half;
-          vec8 bd = lds_col8<T>(do_lds, kRowStride, row0, 32 * wave, lane);
-          vec8 bq = lds_col8<T>(q_lds, kRowStride, row0, 32 * wave, lane);
+          vec8 bd = lds_col8<T>(do_lds, kRowStride, row0, 32 * ct, lane);
+          vec8 bq = lds_col8<T>(q_lds, kRowStride, row0, 32 * ct, lane);
 #pragma unroll
-          for (int mt = 0; mt < 2; mt++) {
-            vec8 ap = lds_col8<T>(p_lds, kPStride, row0, 32 * mt, lane);
+          for (int mt = 0; mt < kMT; mt++) {
+            vec8 ap = lds_col8<T>(p_lds, kPStride, row0, 32 * (mt0 + mt), lane);
             dvacc[mt] = Elem<T>::mfma(ap, bd, dvacc[mt]);
-            vec8 az = lds_col8<T>(dz_lds, kPStride, row0, 32 * mt, lane);
+            vec8 az = lds_col8<T>(dz_lds, kPStride, row0, 32 * (mt0 + mt), lane);
             dkacc[mt] = Elem<T>::mfma(az, bq, dkacc[mt]);
           }
         }
       }
       __syncthreads();
     }
-    // acc[mt][r]: key j0 + 32*mt + 8*(r/4) + 4*half + r%4, column 32*wave + col.
+    // acc[mt][r]: key j0 + 32*(mt0 + mt) + 8*(r/4) + 4*half + r%4, column 32*ct + col.
     T* dkb = (T*)p.dk.ptr + tile.seq_id * p.dk.sb + head * p.dk.sh + tok0 * p.dk.st;
     T* dvb = (T*)p.dv.ptr + tile.seq_id * p.dv.sb + head * p.dv.sh + tok0 * p.dv.st;
-    const int d = 32 * wave + col;
+    const int d = 32 * ct + col;
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++)
+    for (int mt = 0; mt < kMT; mt++)
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const int key = j0 + 32 * mt + 8 * (r >> 2) + 4 * half + (r & 3);
+        const int key = j0 + 32 * (mt0 + mt) + 8 * (r >> 2) + 4 * half + (r & 3);
         if (key < L) {
           dkb[(int64_t)key * p.dk.st + d] = (T)(dkacc[mt][r] * p.logit_scale);
           dvb[(int64_t)key * p.dv.st + d] = (T)dvacc[mt][r];
@@ -393,15 +395,15 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
   }
 }
 
-template <typename T>
+template <typename T, int DH>
 static hipError_t launch_dkv3(const BwdParams& p, int max_tiles, hipStream_t stream) {
-  const size_t lds_bytes = (size_t)Dkv3Lds<128>::kElems * sizeof(T);
+  const size_t lds_bytes = (size_t)Dkv3Lds<DH>::kElems * sizeof(T);
   // The tile set exceeds the default 64 KB dynamic-LDS cap; the attribute is per device and cheap to set.
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv3_kernel<T>),
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv3_kernel<T, DH>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (e != hipSuccess) return e;
   const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kDkv3Threads);
-  hipLaunchKernelGGL((bwd_dkv3_kernel<T>), grid, block, lds_bytes, stream, p);
+  hipLaunchKernelGGL((bwd_dkv3_kernel<T, DH>), grid, block, lds_bytes, stream, p);
   return hipGetLastError();
 }
 
@@ -419,8 +421,8 @@ static hipError_t launch_one(const BwdParams& p, int max_tiles, hipStream_t stre
 
 template <typename T>
 static hipError_t launch_t(const BwdParams& p, int max_tiles, hipStream_t stream) {
-  if (p.vec_ok && p.head_dim == 128) return launch_dkv3<T>(p, max_tiles, stream);
-  if (p.vec_ok && p.head_dim == 64) return launch_one<T, 64, true>(p, max_tiles, stream);
+  if (p.vec_ok && p.head_dim == 128) return launch_dkv3<T, 128>(p, max_tiles, stream);
+  if (p.vec_ok && p.head_dim == 64) return launch_dkv3<T, 64>(p, max_tiles, stream);
   return p.head_dim <= 64 ? launch_one<T, 64, false>(p, max_tiles, stream) : launch_one<T, 128, false>(p, max_tiles, stream);
 }
 

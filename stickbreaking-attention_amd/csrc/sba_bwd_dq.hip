@@ -164,7 +164,7 @@ static hipError_t launch_t(const BwdParams& p, int max_tiles, hipStream_t stream
   if (p.vec_ok && p.head_dim == 128) {
     hipLaunchKernelGGL((bwd_dq_kernel<T, 128, true, 32>), grid, block, 0, stream, p);
   } else if (p.vec_ok && p.head_dim == 64) {
-    hipLaunchKernelGGL((bwd_dq_kernel<T, 64, true, 64>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((bwd_dq_kernel<T, 64, true, 32>), grid, block, 0, stream, p);
   } else if (p.head_dim <= 64) {
     hipLaunchKernelGGL((bwd_dq_kernel<T, 64, false, 64>), grid, block, 0, stream, p);
   } else {
