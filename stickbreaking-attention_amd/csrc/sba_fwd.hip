@@ -102,26 +102,28 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
     }
 
     // This lane's N keys are j0 + N*half + R, R = 16*mt + r, swept from R = N-1 down.
-    //   t[R] = e[R] * prod_{R' >= R} 1/(1+e[R'])   (the weight of key R up to the product carried into the tile)
-    // Hidden keys (diagonal tiles only) get e = 0: factor 1, weight 0.
+    //   t[R] = sigma[R] * prod_{R' > R} (1 - sigma[R']) = run_before - run_after   with run *= 1/(1+e[R])
+    // (the weight of key R up to the product carried into the tile).  The difference form needs neither sigma
+    // nor a clamp: e = inf gives a factor 0 and the whole remaining stick as weight; its absolute error is one
+    // ulp of the running product.  Hidden keys (diagonal tiles only) get e = 0: factor 1, weight 0.
     float t[N];
     float run = 1.f;
     if (diagonal) {
       const int lim = qi + ac - j0 - N * half;                // key R is visible iff R < lim
 #pragma unroll
       for (int R = N - 1; R >= 0; --R) {
-        float x = fast_min(s[R >> 4][R & 15] * p.scale_log2, kExpClamp);
+        float x = s[R >> 4][R & 15] * p.scale_log2;
         x = (R < lim) ? x : -INFINITY;
-        const float e = fast_exp2(x);
-        run *= fast_rcp(1.f + e);
-        t[R] = e * run;
+        const float before = run;
+        run *= fast_rcp(1.f + fast_exp2(x));
+        t[R] = before - run;
       }
     } else {
 #pragma unroll
       for (int R = N - 1; R >= 0; --R) {
-        const float e = fast_exp2(fast_min(s[R >> 4][R & 15] * p.scale_log2, kExpClamp));
-        run *= fast_rcp(1.f + e);
-        t[R] = e * run;
+        const float before = run;
+        run *= fast_rcp(1.f + fast_exp2(s[R >> 4][R & 15] * p.scale_log2));
+        t[R] = before - run;
       }
     }
     const float oth = other_half(run, half);
