@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 1
+#define SBA_VERSION 2
 
 typedef enum SbaDtype { SBA_BF16 = 0, SBA_F32 = 1, SBA_F16 = 2 } SbaDtype;
 
@@ -82,8 +82,8 @@ typedef struct SbaArgs {
   SbaVector rem;               /* forward output, dtype of q: 1 - sum_j A_ij */
   float* row_stat;             /* forward output, fp32, contiguous (H, T) / (B, H, L): log2(rem) */
   float* carry;                /* forward output (optional, NULL when no backward will follow) and backward input:
-                                  for every row and every 64-key tile the row sweeps, the product of (1 - sigma)
-                                  over the keys between that tile and the row.  sba_workspace_bytes sizes it. */
+                                  for every row and every 32-key sub-tile the row sweeps, the product of (1 - sigma)
+                                  over the keys between that sub-tile and the row.  sba_workspace_bytes sizes it. */
 
   SbaTensor d_o;               /* backward input: gradient of o */
   SbaVector d_rem;             /* backward input: gradient of rem (ptr may be NULL = zeros) */
@@ -96,6 +96,12 @@ typedef struct SbaArgs {
                                   caller can time the kernels separately.  sba_fwd records [0] before and [1] after
                                   the attention kernel (the scheduler kernel runs before [0]); sba_bwd records [0]
                                   before the dQ kernel, [1] between the dQ and dK/dV kernels and [2] after. */
+  int32_t add_remainder;       /* 1: the forward writes o + rem * v instead of o, the step every caller of the
+                                  reference applies to its outputs (tests/test_varlen.py:103, tests/test_attn.py:67).
+                                  The backward then takes d_o as the gradient of that sum and d_rem as the
+                                  gradient that reaches rem directly, needs row_stat (as the forward wrote it) as an
+                                  input, and returns dv including rem * d_o. */
+  int32_t reserved0;           /* must be 0 */
 } SbaArgs;
 
 /* ABI version of this header (SBA_VERSION) the library was built against. */
@@ -122,7 +128,7 @@ int sba_workspace_bytes(const SbaArgs* args, size_t* fwd_bytes, size_t* bwd_byte
 int sba_fwd(const SbaArgs* args);
 
 /*
- * Backward: fills dq, dk, dv from q, k, v, carry, d_o, d_rem.  Every element of dq, dk, dv is written
+ * Backward: fills dq, dk, dv from q, k, v, carry, d_o, d_rem (and row_stat when add_remainder is set).  Every element of dq, dk, dv is written
  * exactly once (no zero-fill needed, no atomics, no locks).
  * Replaces `_compileable_backward` (stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:541-640,
  * custom op "varlen_bwd") and (stickbreaking_attention/sb_attn/sb_bwd.py:207-296, custom op

@@ -202,6 +202,26 @@ def dense_backward_autograd(q, k, v, cu_seqlens, do, drem, scale=None, zero_star
     return o.detach(), rem.detach(), q.grad, k.grad, v.grad
 
 
+def with_remainder(outputs, v, do=None):
+    """The step callers of the reference apply to its outputs, ``o + rem[..., None] * v``
+    (tests/test_varlen.py:103, tests/test_attn.py:67), applied to an (o, rem[, dq, dk, dv]) tuple that was
+    evaluated for the gradients ``(do, drem + (do * v).sum(-1))``: y = o + rem v has
+    d/d(o) = do, d/d(rem) = drem + do . v, and dv gains rem * do."""
+    o, rem = outputs[0], outputs[1]
+    vf = v.to(o.dtype)
+    y = o + rem[..., None] * vf
+    if len(outputs) == 2:
+        return y, rem
+    dq, dk, dv = outputs[2:]
+    return y, rem, dq, dk, dv + rem[..., None] * do.to(o.dtype)
+
+
+def remainder_drem(do, drem, v):
+    """Gradient that reaches ``rem`` when the output is ``o + rem[..., None] * v``."""
+    extra = (do.double() * v.double()).sum(-1)
+    return extra if drem is None else drem.double() + extra
+
+
 # --------------------------------------------------------------------------------------------
 # Work accounting shared by tests and the benchmark
 # --------------------------------------------------------------------------------------------

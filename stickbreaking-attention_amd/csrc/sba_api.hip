@@ -23,7 +23,7 @@ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 struct Layout {
   int64_t max_q_tiles, max_k_tiles, carry_slots_per_head;
-  size_t off_counts, off_q_tiles, off_k_tiles, off_carry_base, off_prefix;
+  size_t off_counts, off_q_tiles, off_k_tiles, off_carry_base, off_prefix, off_drem;
   size_t fwd_bytes, bwd_bytes, carry_bytes;
 };
 
@@ -54,6 +54,8 @@ int plan(const SbaArgs* a, Layout* out) {
   L.off_k_tiles = off;     off = align_up(off + (size_t)L.max_k_tiles * sizeof(sba::Tile), 256);
   L.carry_bytes = align_up((size_t)L.carry_slots_per_head * a->num_heads * sizeof(float), 256);
   L.off_prefix = off;      off += L.carry_bytes;
+  // d_rem + d_o . v per row (fp32), used when the remainder term is fused
+  L.off_drem = off;        off = align_up(off + (size_t)a->num_heads * (size_t)T * (fixed ? (size_t)B : 1) * sizeof(float), 256);
   L.bwd_bytes = off;
   *out = L;
   return SBA_OK;
@@ -162,6 +164,7 @@ int sba_fwd(const SbaArgs* a) {
   p.head_dim = a->head_dim;
   p.scale_log2 = (float)((double)a->logit_scale * kLog2e);
   p.attend_current = a->attend_current ? 1 : 0;
+  p.add_rem = a->add_remainder ? 1 : 0;
   const int64_t max_rows = (a->max_seqlen > 0 && a->max_seqlen < a->total_tokens) ? a->max_seqlen : a->total_tokens;
   bool v16 = (a->head_dim % (16 / (int)es)) == 0;
   for (const SbaTensor* t : {&a->q, &a->k, &a->v}) v16 = v16 && vec16(*t, es, fixed, max_rows);
@@ -188,6 +191,7 @@ int sba_bwd(const SbaArgs* a) {
       (st = check_tensor(a->dv, true, fixed)))
     return st;
   if (!a->carry) return SBA_ERR_NULL;
+  if (a->add_remainder && !a->row_stat) return SBA_ERR_NULL;
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
     if (t->ptr && ((uintptr_t)t->ptr % es)) return SBA_ERR_ALIGN;
   if (!a->workspace || ((uintptr_t)a->workspace & 255) || a->workspace_bytes < L.bwd_bytes) return SBA_ERR_WORKSPACE;
@@ -212,6 +216,11 @@ int sba_bwd(const SbaArgs* a) {
   p.scale_log2 = (float)((double)a->logit_scale * kLog2e);
   p.logit_scale = a->logit_scale;
   p.attend_current = a->attend_current ? 1 : 0;
+  p.add_rem = a->add_remainder ? 1 : 0;
+  p.row_stat = a->row_stat;
+  p.stat_sb = fixed ? (int64_t)a->num_heads * a->total_tokens : 0;
+  p.stat_sh = a->total_tokens;
+  p.drem_eff = (float*)(ws + L.off_drem);
   const int64_t max_rows = (a->max_seqlen > 0 && a->max_seqlen < a->total_tokens) ? a->max_seqlen : a->total_tokens;
   bool v16 = (a->head_dim % (16 / (int)es)) == 0;
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})

@@ -113,9 +113,8 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
       for (int i = 0; i < 16; i++) { pk[i] = 0; dzk[i] = 0; }
     } else {
       const bool diagonal = (j0 + kBlockK - 1) > (w_first - 1 + ac) || w_last >= L;
-      float drem = 0.f;
-      if (row_ok && p.d_rem.ptr)
-        drem = (float)((const T*)p.d_rem.ptr)[tile.seq_id * p.d_rem.sb + head * p.d_rem.sh + (tok0 + qi) * p.d_rem.st];
+      // gradient of rem per row, as the dQ kernel left it (d_rem, plus d_o . v when the remainder term is fused)
+      const float drem = row_ok ? p.drem_eff[tile.seq_id * p.stat_sb + head * p.stat_sh + tok0 + qi] : 0.f;
       const float prod_in = carry[qi], prefix_in = prefix[qi];
       f32x16 s[2], dp[2];
 #pragma unroll
@@ -177,7 +176,10 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
       const int key = j0 + 32 * out_mt[b] + 8 * (r >> 2) + 4 * half + (r & 3);
       if (key < L && d < D) {
         dkb[(int64_t)key * p.dk.st + d] = (T)(dkacc[b][r] * p.logit_scale);
-        dvb[(int64_t)key * p.dv.st + d] = (T)dvacc[b][r];
+        float dvv = dvacc[b][r];
+        if (p.add_rem)     // the remainder term o += rem * v contributes rem_j * d_o_j to dv_j
+          dvv += fast_exp2(p.row_stat[tile.seq_id * p.stat_sb + head * p.stat_sh + tok0 + key]) * (float)dob[(int64_t)key * p.d_o.st + d];
+        dvb[(int64_t)key * p.dv.st + d] = (T)dvv;
       }
     }
   }
@@ -238,7 +240,6 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
     const T* kb = (const T*)p.k.ptr + tile.seq_id * p.k.sb + head * p.k.sh + tok0 * p.k.st;
     const T* vb = (const T*)p.v.ptr + tile.seq_id * p.v.sb + head * p.v.sh + tok0 * p.v.st;
     const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
-    const T* dremb = p.d_rem.ptr ? (const T*)p.d_rem.ptr + tile.seq_id * p.d_rem.sb + head * p.d_rem.sh + tok0 * p.d_rem.st : nullptr;
     const int64_t slot0 = (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] +
                           carry_offset(2 * jt + group, n_qt) - (int64_t)kBlockQ * (jt >> 1);      // + row
     const float* carry = p.carry + slot0;
@@ -255,11 +256,11 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
       }
     }
     // Per-row scalars (drem, product above the sub-tile, C below it), fetched one step ahead.
-    T n_drem = (T)0.f;
-    float n_prod = 1.f, n_prefix = 0.f;
+    const float* drem_eff = p.drem_eff + tile.seq_id * p.stat_sb + head * p.stat_sh + tok0;
+    float n_drem = 0.f, n_prod = 1.f, n_prefix = 0.f;
     auto fetch_row_scalars = [&](int row0) {
       const int r = row0 + rg * 32 + col;
-      n_drem = (dremb && r < L) ? dremb[(int64_t)r * p.d_rem.st] : (T)0.f;
+      n_drem = r < L ? drem_eff[r] : 0.f;      // as the dQ kernel left it: d_rem (+ d_o . v with the remainder term)
       n_prod = carry[r];
       n_prefix = prefix[r];
     };
@@ -272,7 +273,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
         const T* do_lds = q_lds + Lds::kQdoTile;
         T* p_lds = lds + Lds::kP + (t & 1) * 2 * Lds::kPTile;
         T* dz_lds = p_lds + Lds::kPTile;
-        const float drem = (float)n_drem, prod_in = n_prod, prefix_in = n_prefix;
+        const float drem = n_drem, prod_in = n_prod, prefix_in = n_prefix;
         if (t + 1 < n_steps) fetch_row_scalars(q0 + kDkvRows);
         const int w_first = q0 + rg * 32, w_last = w_first + 31;
         const int qi = w_first + col;
@@ -389,7 +390,10 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
         const int key = j0 + 32 * (mt0 + mt) + 8 * (r >> 2) + 4 * half + (r & 3);
         if (key < L) {
           dkb[(int64_t)key * p.dk.st + d] = (T)(dkacc[mt][r] * p.logit_scale);
-          dvb[(int64_t)key * p.dv.st + d] = (T)dvacc[mt][r];
+          float dvv = dvacc[mt][r];
+          if (p.add_rem)     // the remainder term o += rem * v contributes rem_j * d_o_j to dv_j
+            dvv += fast_exp2(p.row_stat[tile.seq_id * p.stat_sb + head * p.stat_sh + tok0 + key]) * (float)dob[(int64_t)key * p.d_o.st + d];
+          dvb[(int64_t)key * p.dv.st + d] = (T)dvv;
         }
       }
   }

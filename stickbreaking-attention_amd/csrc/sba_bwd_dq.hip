@@ -54,6 +54,19 @@ __global__ __launch_bounds__(kThreads, KT == 32 ? 2 : 1) void bwd_dq_kernel(BwdP
   float drem = 0.f;
   if (row_ok && p.d_rem.ptr)
     drem = (float)((const T*)p.d_rem.ptr)[tile.seq_id * p.d_rem.sb + head * p.d_rem.sh + (tok0 + qi) * p.d_rem.st];
+  if (p.add_rem) {
+    // The forward wrote o + rem * v: the gradient reaching rem is d_rem + d_o . v_i.
+    float dot = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < kSteps; kk++) {
+      const vec8 vv = as_vec8<T>(load_row8<T, kFast>(vb + (int64_t)qi * p.v.st, 16 * kk + 8 * half, D, row_ok));
+#pragma unroll
+      for (int t = 0; t < 8; t++) dot = fmaf((float)dof[kk][t], (float)vv[t], dot);
+    }
+    drem += dot + other_half(dot, half);
+  }
+  // The dK/dV kernel reads the gradient of rem back from this fp32 plane (one value per row).
+  if (half == 0 && row_ok) p.drem_eff[tile.seq_id * p.stat_sb + head * p.stat_sh + tok0 + qi] = drem;
   float prefix = 0.f;      // sum of g over the keys already swept (both half-waves hold the same value)
 
   const int last_row = min(q0 + kBlockQ, L) - 1;

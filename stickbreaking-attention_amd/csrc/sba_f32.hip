@@ -98,6 +98,10 @@ __global__ __launch_bounds__(kThreads) void fwd_f32_kernel(FwdParams p) {
         if (lane + 64 < D) o1 = fmaf(at, vrow[lane + 64], o1);
       }
     }
+    if (p.add_rem) {                                         // o + rem * v
+      if (lane < D) o0 = fmaf(prod, vb[(int64_t)i * p.v.st + lane], o0);
+      if (lane + 64 < D) o1 = fmaf(prod, vb[(int64_t)i * p.v.st + lane + 64], o1);
+    }
     if (lane < D) ob[(int64_t)i * p.o.st + lane] = o0;
     if (lane + 64 < D) ob[(int64_t)i * p.o.st + lane + 64] = o1;
     if (lane == 0) {
@@ -151,6 +155,15 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_kernel(BwdParams p) {
   const int n_steps = (wg_last_key < 0 || wg_row0 >= L) ? 0 : wg_last_key / kF32Keys + 1;
   for (int idx = threadIdx.x; idx < kF32Rows * kMaxD; idx += kThreads) (&lds.dq[0][0])[idx] = 0.f;
   float prefix_row = 0.f;      // lane r (< rows per wave) holds the running prefix sum C of this wave's row r
+  if (p.add_rem) {
+    // The forward wrote o + rem * v: dv_i gains rem_i * d_o_i, for every row including those that see no key.
+    for (int r = 0; r < kF32RowsPerWave; r++) {
+      const int i = wg_row0 + wave * kF32RowsPerWave + r;
+      if (i >= L) break;
+      const float rem_i = exp2f(p.row_stat[tile.seq_id * p.stat_sb + head * p.stat_sh + tok0 + i]);
+      for (int d = lane; d < D; d += 64) atomicAdd(&dvb[(int64_t)i * p.dv.st + d], rem_i * dob[(int64_t)i * p.d_o.st + d]);
+    }
+  }
 
   for (int c = 0; c < n_steps; ++c) {
     const int j0 = c * kF32Keys;
@@ -164,7 +177,15 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_kernel(BwdParams p) {
         lds.q[wave][d] = qb[(int64_t)i * p.q.st + d];
         lds.d_o[wave][d] = dob[(int64_t)i * p.d_o.st + d];
       }
-      const float drem = p.d_rem.ptr ? ((const float*)p.d_rem.ptr)[tile.seq_id * p.d_rem.sb + head * p.d_rem.sh + (tok0 + i) * p.d_rem.st] : 0.f;
+      float drem = p.d_rem.ptr ? ((const float*)p.d_rem.ptr)[tile.seq_id * p.d_rem.sb + head * p.d_rem.sh + (tok0 + i) * p.d_rem.st] : 0.f;
+      if (p.add_rem) {
+        // The forward wrote o + rem * v: the gradient reaching rem gains d_o . v_i.
+        const float* vrow = vb + (int64_t)i * p.v.st;
+        float dot = 0.f;
+        for (int d = lane; d < D; d += 64) dot = fmaf(lds.d_o[wave][d], vrow[d], dot);
+        for (int m = 32; m >= 1; m >>= 1) dot += __shfl_xor(dot, m);
+        drem += dot;
+      }
       const float prod_in = carry[carry_offset(2 * c + 1, n_qt) + (i - kBlockQ * (c >> 1))];
       const float prefix_in = wave_bcast(prefix_row, r);
       const int j = j0 + lane;

@@ -149,13 +149,30 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
 
   // Epilogue.  oacc[dt][r]: query row 8*(r/4) + 4*half + r%4 of this wave, column 32*dt + col.
   T* ob = (T*)p.o.ptr + tile.seq_id * p.o.sb + head * p.o.sh + (int64_t)tile.seq_start * p.o.st;
-#pragma unroll
-  for (int dt = 0; dt < kDTiles; dt++) {
-    const int d = 32 * dt + col;
+  if (p.add_rem) {
+    // o + rem * v (the step callers of the reference apply to its outputs, tests/test_varlen.py:103): the row's
+    // remainder is held by the lane whose query it is.
 #pragma unroll
     for (int r = 0; r < 16; r++) {
-      const int row = w_first + 8 * (r >> 2) + 4 * half + (r & 3);
-      if (row < L && d < D) ob[(int64_t)row * p.o.st + d] = (T)oacc[dt][r];
+      const int lr = 8 * (r >> 2) + 4 * half + (r & 3);
+      const int row = w_first + lr;
+      const float rem_row = __shfl(prod, lr);
+#pragma unroll
+      for (int dt = 0; dt < kDTiles; dt++) {
+        const int d = 32 * dt + col;
+        if (row < L && d < D)
+          ob[(int64_t)row * p.o.st + d] = (T)(oacc[dt][r] + rem_row * (float)vb[(int64_t)row * p.v.st + d]);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int dt = 0; dt < kDTiles; dt++) {
+      const int d = 32 * dt + col;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int row = w_first + 8 * (r >> 2) + 4 * half + (r & 3);
+        if (row < L && d < D) ob[(int64_t)row * p.o.st + d] = (T)oacc[dt][r];
+      }
     }
   }
   if (half == 0 && qi < L) {

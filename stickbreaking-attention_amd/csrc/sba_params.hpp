@@ -49,6 +49,7 @@ struct FwdParams {
   float scale_log2;            // logit_scale * log2(e)
   int32_t attend_current;
   int32_t vec_ok;              // all row strides / base pointers allow 16-byte accesses and head_dim % 8 == 0
+  int32_t add_rem;             // write o + rem * v
 };
 
 struct BwdParams {
@@ -66,6 +67,12 @@ struct BwdParams {
   float logit_scale;
   int32_t attend_current;
   int32_t vec_ok;
+  // Fused remainder term (the forward wrote o + rem * v): d_rem_eff = d_rem + d_o . v per row, dv += rem * d_o.
+  int32_t add_rem;
+  const float* row_stat;       // log2(rem), fp32 [batch][head][token]
+  int64_t stat_sb, stat_sh;
+  float* drem_eff;             // workspace, indexed like row_stat: the gradient of rem per row in fp32 (d_rem, plus
+                               // d_o . v when add_rem), written by the dQ kernel and read by the dK/dV kernel
 };
 
 // Carry slots.  Carries are kept per (row, 32-key sub-tile): sub-tile U covers keys 32U .. 32U+31 of the

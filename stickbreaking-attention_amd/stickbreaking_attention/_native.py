@@ -14,6 +14,7 @@ import torch
 from .utils import custom_op
 
 _LIB_NAME = "libsba.so"
+ABI_VERSION = 2          # SBA_VERSION of include/sba.h this binding mirrors
 _lib = None
 # Optional ctypes array of hipEvent_t handed to the next calls as SbaArgs.trace_events (benchmarks only).
 TRACE_EVENTS = None
@@ -42,6 +43,7 @@ class SbaArgs(ctypes.Structure):
         ("d_o", SbaTensor), ("d_rem", SbaVector), ("dq", SbaTensor), ("dk", SbaTensor), ("dv", SbaTensor),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t), ("stream", ctypes.c_void_p),
         ("trace_events", ctypes.POINTER(ctypes.c_void_p)),
+        ("add_remainder", ctypes.c_int32), ("reserved0", ctypes.c_int32),
     ]
 
 
@@ -70,8 +72,8 @@ def lib():
             fn = getattr(handle, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.POINTER(SbaArgs)]
-        if handle.sba_version() != 1:
-            raise RuntimeError(f"{path}: ABI version {handle.sba_version()} != 1")
+        if handle.sba_version() != ABI_VERSION:
+            raise RuntimeError(f"{path}: ABI version {handle.sba_version()} != {ABI_VERSION}")
         _lib = handle
     return _lib
 
@@ -157,10 +159,12 @@ def carry_elems(num_heads: int, total_tokens: int, num_seqs: int, max_seqlen, fi
     return nbytes // 4
 
 
-def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, o, rem, neg_log_acc, carry):
+def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, add_remainder, o, rem,
+                neg_log_acc, carry):
     fixed = cu_seqlens is None
     with torch.cuda.device(q.device):
         a = _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current)
+        a.add_remainder = 1 if add_remainder else 0
         a.q, a.k, a.v, a.o = (_tensor(t, fixed) for t in (q, k, v, o))
         a.rem = _vector(rem, fixed)
         a.row_stat = neg_log_acc.data_ptr()
@@ -175,10 +179,13 @@ def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scal
         _check(lib().sba_fwd(ctypes.byref(a)), "sba_fwd")
 
 
-def _launch_bwd(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, dq, dk, dv):
+def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current,
+                add_remainder, dq, dk, dv):
     fixed = cu_seqlens is None
     with torch.cuda.device(q.device):
         a = _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current)
+        a.add_remainder = 1 if add_remainder else 0
+        a.row_stat = neg_log_acc.data_ptr() if neg_log_acc.numel() > 0 else None
         a.q, a.k, a.v, a.d_o, a.dq, a.dk, a.dv = (_tensor(t, fixed) for t in (q, k, v, do, dq, dk, dv))
         a.d_rem = _vector(drem, fixed)
         a.carry = carry.data_ptr()
@@ -195,33 +202,39 @@ def _launch_bwd(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_s
 # only".
 @custom_op("varlen_fwd", mutates_args={"o", "rem", "neg_log_acc", "carry"})
 def varlen_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor, cu_has_leading_zero: bool,
-               max_seqlens: int, logit_scale: float, attend_current: bool, o: torch.Tensor, rem: torch.Tensor,
-               neg_log_acc: torch.Tensor, carry: torch.Tensor) -> None:
-    _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlens, logit_scale, attend_current, o, rem, neg_log_acc, carry)
+               max_seqlens: int, logit_scale: float, attend_current: bool, add_remainder: bool, o: torch.Tensor,
+               rem: torch.Tensor, neg_log_acc: torch.Tensor, carry: torch.Tensor) -> None:
+    _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlens, logit_scale, attend_current, add_remainder, o, rem,
+                neg_log_acc, carry)
 
 
 @custom_op("varlen_bwd", mutates_args={"dq", "dk", "dv"})
 def varlen_bwd(do: torch.Tensor, drem: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, carry: torch.Tensor,
-               cu_seqlens: torch.Tensor, cu_has_leading_zero: bool, max_seqlens: int, logit_scale: float,
-               attend_current: bool, dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor) -> None:
-    _launch_bwd(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlens, logit_scale, attend_current, dq, dk, dv)
+               neg_log_acc: torch.Tensor, cu_seqlens: torch.Tensor, cu_has_leading_zero: bool, max_seqlens: int,
+               logit_scale: float, attend_current: bool, add_remainder: bool, dq: torch.Tensor, dk: torch.Tensor,
+               dv: torch.Tensor) -> None:
+    _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leading_zero, max_seqlens, logit_scale, attend_current,
+                add_remainder, dq, dk, dv)
 
 
 @custom_op("attn_fwd", mutates_args={"o", "rem", "neg_log_acc", "carry"})
-def attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_scale: float, attend_current: bool,
+def attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_scale: float, attend_current: bool, add_remainder: bool,
              o: torch.Tensor, rem: torch.Tensor, neg_log_acc: torch.Tensor, carry: torch.Tensor) -> None:
-    _launch_fwd(q, k, v, None, False, q.size(2), logit_scale, attend_current, o, rem, neg_log_acc, carry)
+    _launch_fwd(q, k, v, None, False, q.size(2), logit_scale, attend_current, add_remainder, o, rem, neg_log_acc, carry)
 
 
 @custom_op("attn_bwd", mutates_args={"dq", "dk", "dv"})
 def attn_bwd(do: torch.Tensor, drem: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, carry: torch.Tensor,
-             logit_scale: float, attend_current: bool, dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor) -> None:
-    _launch_bwd(do, drem, q, k, v, carry, None, False, q.size(2), logit_scale, attend_current, dq, dk, dv)
+             neg_log_acc: torch.Tensor, logit_scale: float, attend_current: bool, add_remainder: bool, dq: torch.Tensor,
+             dk: torch.Tensor, dv: torch.Tensor) -> None:
+    _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, None, False, q.size(2), logit_scale, attend_current, add_remainder,
+                dq, dk, dv)
 
 
-def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, want_carry):
+def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, want_carry, add_remainder=False):
     """Launch the forward.  Returns (o, rem, row_stat, carry or None).  Packed mode when cu_seqlens is given.
-    ``carry`` is the buffer the backward needs; it is only produced when ``want_carry``."""
+    ``carry`` is the buffer the backward needs; it is only produced when ``want_carry``.  With ``add_remainder`` the
+    first output is ``o + rem[..., None] * v``."""
     _require_gpu(q, k, v)
     fixed = cu_seqlens is None
     q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)
@@ -240,15 +253,17 @@ def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, a
             n_carry = carry_elems(q.size(0), q.size(1), cu_seqlens.numel() - (1 if cu_has_leading_zero else 0), max_seqlen, False)
     carry = torch.empty(n_carry, dtype=torch.float32, device=q.device)
     if fixed:
-        attn_fwd(q, k, v, float(logit_scale), bool(attend_current), o, rem, row_stat, carry)
+        attn_fwd(q, k, v, float(logit_scale), bool(attend_current), bool(add_remainder), o, rem, row_stat, carry)
     else:
         varlen_fwd(q, k, v, cu_seqlens, bool(cu_has_leading_zero), int(max_seqlen) if max_seqlen else 0, float(logit_scale),
-                   bool(attend_current), o, rem, row_stat, carry)
+                   bool(attend_current), bool(add_remainder), o, rem, row_stat, carry)
     return o, rem, row_stat, (carry if want_carry else None)
 
 
-def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current):
-    """Launch the backward.  Returns (dq, dk, dv)."""
+def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current,
+             row_stat=None, add_remainder=False):
+    """Launch the backward.  Returns (dq, dk, dv).  ``row_stat`` (the forward's third output) is needed when the
+    forward ran with ``add_remainder``."""
     _require_gpu(q, k, v, do, drem, carry)
     fixed = cu_seqlens is None
     do = rows_contiguous(do)
@@ -258,9 +273,13 @@ def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seql
         drem = torch.zeros(q.shape[:-1], dtype=q.dtype, device=q.device)
     elif drem.dtype != q.dtype:
         drem = drem.to(q.dtype)
+    if add_remainder and row_stat is None:
+        raise ValueError("the backward of add_remainder needs the forward's row_stat")
+    if row_stat is None:
+        row_stat = torch.empty(0, dtype=torch.float32, device=q.device)
     if fixed:
-        attn_bwd(do, drem, q, k, v, carry, float(logit_scale), bool(attend_current), dq, dk, dv)
+        attn_bwd(do, drem, q, k, v, carry, row_stat, float(logit_scale), bool(attend_current), bool(add_remainder), dq, dk, dv)
     else:
-        varlen_bwd(do, drem, q, k, v, carry, cu_seqlens, bool(cu_has_leading_zero), int(max_seqlen) if max_seqlen else 0,
-                   float(logit_scale), bool(attend_current), dq, dk, dv)
+        varlen_bwd(do, drem, q, k, v, carry, row_stat, cu_seqlens, bool(cu_has_leading_zero),
+                   int(max_seqlen) if max_seqlen else 0, float(logit_scale), bool(attend_current), bool(add_remainder), dq, dk, dv)
     return dq, dk, dv

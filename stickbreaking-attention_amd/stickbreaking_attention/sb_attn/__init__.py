@@ -14,28 +14,31 @@ from .. import _native
 
 class StickBreakingAttention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, inv_temp, attend_current=False):
+    def forward(ctx, q, k, v, inv_temp, attend_current=False, add_remainder=False):
         need_grad = any(ctx.needs_input_grad[:3])
         o, rem, row_stat, carry = _native.forward(q, k, v, None, False, q.size(2), inv_temp, attend_current,
-                                                 want_carry=need_grad)
-        ctx.save_for_backward(q, k, v, carry)
+                                                 want_carry=need_grad, add_remainder=add_remainder)
+        ctx.save_for_backward(q, k, v, carry, row_stat if add_remainder else None)
+        ctx.add_remainder = add_remainder
         ctx.logit_scale = inv_temp
         ctx.attend_current = attend_current
         return o, rem
 
     @staticmethod
     def backward(ctx, do, drem):
-        q, k, v, carry = ctx.saved_tensors
+        q, k, v, carry, row_stat = ctx.saved_tensors
         dq, dk, dv = _native.backward(do, drem, q, k, v, carry, None, False, q.size(2),
-                                      ctx.logit_scale, ctx.attend_current)
-        return dq, dk, dv, None, None
+                                      ctx.logit_scale, ctx.attend_current, row_stat=row_stat, add_remainder=ctx.add_remainder)
+        return dq, dk, dv, None, None, None
 
 
-def sb_attn(q, k, v, inv_temp=None, zero_start=True, attend_current=False):
+def sb_attn(q, k, v, inv_temp=None, zero_start=True, attend_current=False, add_remainder=False):
+    """``add_remainder=True`` returns ``(o + rem[..., None] * v, rem)`` (what tests/test_attn.py:67 forms from the
+    reference's outputs), fused into the kernels' epilogues."""
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
-    return sb_attn_(q, k, v, inv_temp, attend_current=attend_current)
+    return sb_attn_(q, k, v, inv_temp, attend_current=attend_current, add_remainder=add_remainder)
 
 
-def sb_attn_(q, k, v, inv_temp, attend_current):
-    return StickBreakingAttention.apply(q, k, v, inv_temp, attend_current)
+def sb_attn_(q, k, v, inv_temp, attend_current, add_remainder=False):
+    return StickBreakingAttention.apply(q, k, v, inv_temp, attend_current, bool(add_remainder))

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol(native):
     lib = native.lib()
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.sba_version() == 1
+    assert lib.sba_version() == native.ABI_VERSION == 2
     assert lib.sba_strerror(0) == b"ok"
     for code in range(-8, 0):
         assert lib.sba_strerror(code) not in (b"ok", b"unknown status")

@@ -326,6 +326,58 @@ def test_forward_without_grad_skips_carry(gpu_device):
     torch.testing.assert_close(torch.exp2(stat), rem.float(), atol=4e-3, rtol=4e-3)   # row_stat = log2(rem)
 
 
+@pytest.mark.parametrize("label,H,D,lengths,dtype", [
+    ("d128", 2, 128, [1, 5, 64, 65, 300], torch.bfloat16),
+    ("d64", 3, 64, [200, 33, 130], torch.bfloat16),
+    ("d50-unaligned", 2, 50, [100, 77], torch.bfloat16),
+    ("f16", 2, 128, [257], torch.float16),
+    ("fp32", 2, 64, [1, 70, 129], torch.float32),
+])
+@pytest.mark.parametrize("attend_current", [False, True])
+def test_fused_remainder_term(gpu_device, label, H, D, lengths, dtype, attend_current):
+    """add_remainder=True returns o + rem v (what tests/test_varlen.py:103 forms from the reference's outputs) and
+    back-propagates through it: checked against the oracle, and against composing the plain operator with torch."""
+    from stickbreaking_attention import sb_attn_varlen
+
+    host, dev, cu = small_case(H, D, lengths, dtype, seed=31)
+    cu = cu.to(gpu_device)
+    q, k, v = (t.detach().clone().requires_grad_() for t in dev[:3])
+    y, rem = sb_attn_varlen(q, k, v, cu, max(lengths), zero_start=False, attend_current=attend_current, add_remainder=True)
+    got = [y, rem] + list(torch.autograd.grad([y, rem], [q, k, v], [dev[3], dev[4]]))
+    torch.cuda.synchronize()
+    ref = orc.varlen_stream(*host[:3], cu.cpu(), attend_current=attend_current, do=host[3],
+                            drem=orc.remainder_drem(host[3], host[4], host[2]).float(), dtype=torch.float32)
+    ref = orc.with_remainder(ref, host[2], host[3])
+    for n, a, b in zip(NAMES, got, ref):
+        tol_check(n, a, b, dtype, f"remainder {label}")
+    # composition with torch ops on the plain operator's outputs agrees to rounding
+    q2, k2, v2 = (t.detach().clone().requires_grad_() for t in dev[:3])
+    o2, rem2 = sb_attn_varlen(q2, k2, v2, cu, max(lengths), zero_start=False, attend_current=attend_current)
+    y2 = o2.float() + rem2.float()[..., None] * v2.float()
+    g2 = torch.autograd.grad([y2, rem2], [q2, k2, v2], [dev[3].float(), dev[4]])
+    assert torch.equal(rem, rem2)
+    tol = 1e-5 if dtype == torch.float32 else 6e-2
+    for a, b in zip([y] + got[2:], [y2] + list(g2)):
+        assert (a.float() - b.float()).abs().max().item() <= tol * max(1.0, b.abs().max().item())
+
+
+def test_fused_remainder_fixed_length(gpu_device):
+    from stickbreaking_attention import sb_attn
+
+    B, H, L, D = 2, 3, 160, 128
+    g = torch.Generator().manual_seed(33)
+    q, k, v, dy = (torch.randn(B, H, L, D, generator=g).to(torch.bfloat16) for _ in range(4))
+    drem = torch.randn(B, H, L, generator=g).to(torch.bfloat16)
+    qd, kd, vd = (t.to(gpu_device).requires_grad_() for t in (q, k, v))
+    y, rem = sb_attn(qd, kd, vd, add_remainder=True)
+    got = [y, rem] + list(torch.autograd.grad([y, rem], [qd, kd, vd], [dy.to(gpu_device), drem.to(gpu_device)]))
+    torch.cuda.synchronize()
+    ref = orc.fixed_stream(q, k, v, do=dy, drem=orc.remainder_drem(dy, drem, v).float(), dtype=torch.float32)
+    ref = orc.with_remainder(ref, v, dy)
+    for n, a, b in zip(NAMES, got, ref):
+        tol_check(n, a, b, torch.bfloat16, "remainder fixed")
+
+
 def test_torch_compile_graph_matches_eager(gpu_device):
     """Under torch.compile the launchers run as the registered stickbreaking_attention::* operators; outputs and
     gradients must be bit-identical to the eager call.  (aot_eager backend: graph capture and functionalisation
