@@ -77,6 +77,11 @@ SMALL = [
     ("d16", 2, 16, [130, 2]),
     ("d50-unaligned", 2, 50, [100, 77]),
     ("long-2k", 1, 128, [2048]),
+    ("single-token", 1, 128, [1]),
+    ("d1", 2, 1, [5, 3]),
+    ("d127-unaligned", 3, 127, [70, 1, 130]),
+    ("300-singletons", 2, 8, [1] * 300),
+    ("d24-tile-edges", 5, 24, [33, 64, 63, 65, 127, 128, 129]),
 ]
 
 
