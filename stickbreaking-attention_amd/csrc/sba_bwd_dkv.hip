@@ -217,13 +217,69 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
 
-  int head, slot;
-  xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
-  if (slot >= p.counts[1]) return;
-  const Tile tile = p.k_tiles[slot];
+  // Persistent workgroups: LDS allows one workgroup per CU, so a workgroup per key tile would leave every tile's
+  // start-up (tile record, K/V operands, first query tiles) and its final stores exposed.  Each workgroup walks
+  // the tile list with the grid's stride instead; the producers run ahead into the next tile's start-up while the
+  // consumers store the previous tile's results.  The walk keeps the workgroup on one head (and one XCD).
+  const int n_tiles = p.counts[1];
   const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3;
   const bool producer = threadIdx.x < 256;
   const int half = lane >> 5, col = lane & 31;
+  const int ac = p.attend_current;
+  // The `wph` workgroups of a head take the tiles of that head's list (heaviest first) in rounds of wph, in
+  // alternating order, so that every workgroup gets the same share of heavy and light tiles.
+  const int wph = p.wgs_per_head;
+  int head, w;
+  if ((p.num_heads & 7) == 0) {
+    const int hpx = p.num_heads >> 3, r0 = blockIdx.x >> 3;
+    head = (blockIdx.x & 7) * hpx + r0 % hpx;
+    w = r0 / hpx;
+  } else {
+    head = blockIdx.x % p.num_heads;
+    w = blockIdx.x / p.num_heads;
+  }
+  auto slot_of = [&](int round) { return wph * round + ((round & 1) ? wph - 1 - w : w); };
+  auto first_row_block = [&](const Tile& tl) {               // first 64-row step that sees the tile's first key
+    const int first_row = tl.origin + 1 - ac;
+    return first_row < tl.seq_len ? (first_row / kDkvRows) * kDkvRows : tl.seq_len;
+  };
+  // The tile record of the next round is fetched a round ahead; the consumers also request the first query rows
+  // of the next tile before they store the results of the current one.
+  Tile next_tile = p.k_tiles[slot_of(0) < n_tiles ? slot_of(0) : 0];
+  TileCopy<T, DH, kDkvRows, true> cq, cdo;                   // staging registers (consumer waves)
+  auto stage_first = [&](const Tile& tl) {
+    const T* qb = (const T*)p.q.ptr + tl.seq_id * p.q.sb + head * p.q.sh + (int64_t)tl.seq_start * p.q.st;
+    const T* dob = (const T*)p.d_o.ptr + tl.seq_id * p.d_o.sb + head * p.d_o.sh + (int64_t)tl.seq_start * p.d_o.st;
+    const int rb = first_row_block(tl);
+    if (rb < tl.seq_len) {
+      cq.load(make_row_source<T, true>(qb, p.q.st, tl.seq_len, DH), rb);
+      cdo.load(make_row_source<T, true>(dob, p.d_o.st, tl.seq_len, DH), rb);
+    }
+  };
+  // Producer waves: the K and V operands of the next tile's 32-key sub-tile are requested a tile ahead as well.
+  vec8 kf_next[kSteps], vf_next[kSteps];
+  auto load_kv = [&](const Tile& tl) {
+    const T* kb = (const T*)p.k.ptr + tl.seq_id * p.k.sb + head * p.k.sh + (int64_t)tl.seq_start * p.k.st;
+    const T* vb = (const T*)p.v.ptr + tl.seq_id * p.v.sb + head * p.v.sh + (int64_t)tl.seq_start * p.v.st;
+    const int key = tl.origin + 32 * (wave & 1) + mfma_row_to_key32(col);
+    const RowSource<T> ks = make_row_source<T, true>(kb, p.k.st, tl.seq_len, DH), vs = make_row_source<T, true>(vb, p.v.st, tl.seq_len, DH);
+#pragma unroll
+    for (int kk = 0; kk < kSteps; kk++) {       // keys beyond the sequence are outside the buffer and read as zero
+      kf_next[kk] = as_vec8<T>(__builtin_amdgcn_raw_buffer_load_b128(ks.rsrc, key * ks.stride_bytes + (16 * kk + 8 * half) * (int)sizeof(T), 0, 0));
+      vf_next[kk] = as_vec8<T>(__builtin_amdgcn_raw_buffer_load_b128(vs.rsrc, key * vs.stride_bytes + (16 * kk + 8 * half) * (int)sizeof(T), 0, 0));
+    }
+  };
+  // Each role runs its own walk over the same rounds (same tiles, same number of barriers), so that what one role
+  // carries from tile to tile does not occupy registers in the other role's code.
+  if (producer) {
+    if (slot_of(0) < n_tiles) load_kv(next_tile);
+  for (int round = 0; wph * round < n_tiles; ++round) {
+  const int slot = slot_of(round);
+  if (slot >= n_tiles) break;                                // only in the last, partial round
+  const Tile tile = next_tile;
+  const int next_slot = slot_of(round + 1);
+  const bool have_next = next_slot < n_tiles;
+  if (have_next) next_tile = p.k_tiles[next_slot];
   const int L = tile.seq_len, j0 = tile.origin, ac = p.attend_current, D = DH;
   const int64_t tok0 = tile.seq_start;
   const int jt = j0 / kBlockK;
@@ -233,7 +289,6 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
   const int row_begin = first_row < L ? (first_row / kDkvRows) * kDkvRows : L;
   const int n_steps = (L - row_begin + kDkvRows - 1) / kDkvRows;
 
-  if (producer) {
     const int rg = wave >> 1, group = wave & 1;
     const int jb = j0 + 32 * group;          // first key of this wave's sub-tile
     const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
@@ -247,14 +302,8 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
 
     // This sub-tile's K and V as MFMA A operands, stationary in registers (keys beyond the sequence read as zero).
     vec8 kf[kSteps], vf[kSteps];
-    {
-      const int key = jb + mfma_row_to_key32(col);
 #pragma unroll
-      for (int kk = 0; kk < kSteps; kk++) {
-        kf[kk] = as_vec8<T>(load_row8<T, true>(kb + (int64_t)key * p.k.st, 16 * kk + 8 * half, D, key < L));
-        vf[kk] = as_vec8<T>(load_row8<T, true>(vb + (int64_t)key * p.v.st, 16 * kk + 8 * half, D, key < L));
-      }
-    }
+    for (int kk = 0; kk < kSteps; kk++) { kf[kk] = kf_next[kk]; vf[kk] = vf_next[kk]; }
     // Per-row scalars (drem, product above the sub-tile, C below it), fetched one step ahead.
     const float* drem_eff = p.drem_eff + tile.seq_id * p.stat_sb + head * p.stat_sh + tok0;
     float n_drem = 0.f, n_prod = 1.f, n_prefix = 0.f;
@@ -266,6 +315,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
     };
     if (n_steps > 0) fetch_row_scalars(row_begin);
     __syncthreads();
+    if (have_next) load_kv(next_tile);
     for (int t = 0; t <= n_steps; ++t) {
       if (t < n_steps) {
         const int q0 = row_begin + t * kDkvRows;
@@ -287,19 +337,24 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
           f32x16 s[1], dp[1];
 #pragma unroll
           for (int r = 0; r < 16; r++) { s[0][r] = 0.f; dp[0][r] = 0.f; }
-          // All sixteen B operands are requested before the first MFMA: the consumers keep the LDS queue long,
-          // and a read-two / wait / multiply-two schedule pays that queueing latency eight times over.
-          vec8 bq[kSteps], bdo[kSteps];
+          // The B operands are requested in two batches of eight, each before its MFMAs: the consumers keep the LDS
+          // queue long, and a read-two / wait / multiply-two schedule pays that queueing latency eight times over.
+          {
+            vec8 bq[kSteps];
 #pragma unroll
-          for (int kk = 0; kk < kSteps; kk++) {
-            bq[kk] = lds_row8<T>(q_lds, kRowStride, rg * 32 + col, 16 * kk + 8 * half);
-            bdo[kk] = lds_row8<T>(do_lds, kRowStride, rg * 32 + col, 16 * kk + 8 * half);
+            for (int kk = 0; kk < kSteps; kk++) bq[kk] = lds_row8<T>(q_lds, kRowStride, rg * 32 + col, 16 * kk + 8 * half);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < kSteps; kk++) s[0] = Elem<T>::mfma(kf[kk], bq[kk], s[0]);
           }
           __builtin_amdgcn_sched_barrier(0);
+          {
+            vec8 bdo[kSteps];
 #pragma unroll
-          for (int kk = 0; kk < kSteps; kk++) {
-            s[0] = Elem<T>::mfma(kf[kk], bq[kk], s[0]);
-            dp[0] = Elem<T>::mfma(vf[kk], bdo[kk], dp[0]);
+            for (int kk = 0; kk < kSteps; kk++) bdo[kk] = lds_row8<T>(do_lds, kRowStride, rg * 32 + col, 16 * kk + 8 * half);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < kSteps; kk++) dp[0] = Elem<T>::mfma(vf[kk], bdo[kk], dp[0]);
           }
           const int lim = row_ok ? qi + ac - jb - 16 * half : 0;
           float prod_lower, prefix_upper, prefix_next;
@@ -317,7 +372,25 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
       }
       __syncthreads();
     }
+    }  // rounds of the tile walk (producers)
   } else {
+    if (slot_of(0) < n_tiles) stage_first(next_tile);
+  for (int round = 0; wph * round < n_tiles; ++round) {
+  const int slot = slot_of(round);
+  if (slot >= n_tiles) break;                                // only in the last, partial round
+  const Tile tile = next_tile;
+  const int next_slot = slot_of(round + 1);
+  const bool have_next = next_slot < n_tiles;
+  if (have_next) next_tile = p.k_tiles[next_slot];
+  const int L = tile.seq_len, j0 = tile.origin, ac = p.attend_current, D = DH;
+  const int64_t tok0 = tile.seq_start;
+  const int jt = j0 / kBlockK;
+
+  const int first_row = j0 + 1 - ac;                         // first row that sees key j0
+  const int n_qt = (L + kBlockQ - 1) / kBlockQ;
+  const int row_begin = first_row < L ? (first_row / kDkvRows) * kDkvRows : L;
+  const int n_steps = (L - row_begin + kDkvRows - 1) / kDkvRows;
+
     // Output blocks of this consumer wave.  head_dim 128: both 32-key row tiles x columns 32*wave .. +31;
     // head_dim 64: row tile wave/2 x columns 32*(wave%2) .. +31.
     constexpr int kMT = DH == 128 ? 2 : 1;
@@ -333,10 +406,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
     const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
     const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
     const RowSource<T> qsrc = make_row_source<T, true>(qb, p.q.st, L, D), dosrc = make_row_source<T, true>(dob, p.d_o.st, L, D);
-    TileCopy<T, DH, kDkvRows, true> cq, cdo;
-    if (n_steps > 0) {
-      cq.load(qsrc, row_begin);
-      cdo.load(dosrc, row_begin);
+    if (n_steps > 0) {                                       // rows of step 0 were requested a tile ago
       cq.store(lds + Lds::kQ);
       cdo.store(lds + Lds::kQ + Lds::kQdoTile);
       if (n_steps > 1) {
@@ -379,34 +449,51 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
       }
       __syncthreads();
     }
+    if (have_next) stage_first(next_tile);
     // acc[mt][r]: key j0 + 32*(mt0 + mt) + 8*(r/4) + 4*half + r%4, column 32*ct + col.
     T* dkb = (T*)p.dk.ptr + tile.seq_id * p.dk.sb + head * p.dk.sh + tok0 * p.dk.st;
     T* dvb = (T*)p.dv.ptr + tile.seq_id * p.dv.sb + head * p.dv.sh + tok0 * p.dv.st;
     const int d = 32 * ct + col;
+    if (p.add_rem) {
+      // the remainder term o += rem * v contributes rem_j * d_o_j to dv_j
 #pragma unroll
-    for (int mt = 0; mt < kMT; mt++)
+      for (int mt = 0; mt < kMT; mt++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int key = j0 + 32 * (mt0 + mt) + 8 * (r >> 2) + 4 * half + (r & 3);
-        if (key < L) {
-          dkb[(int64_t)key * p.dk.st + d] = (T)(dkacc[mt][r] * p.logit_scale);
-          float dvv = dvacc[mt][r];
-          if (p.add_rem)     // the remainder term o += rem * v contributes rem_j * d_o_j to dv_j
-            dvv += fast_exp2(p.row_stat[tile.seq_id * p.stat_sb + head * p.stat_sh + tok0 + key]) * (float)dob[(int64_t)key * p.d_o.st + d];
-          dvb[(int64_t)key * p.dv.st + d] = (T)dvv;
+        for (int r = 0; r < 16; r++) {
+          const int key = j0 + 32 * (mt0 + mt) + 8 * (r >> 2) + 4 * half + (r & 3);
+          if (key < L)
+            dvacc[mt][r] += fast_exp2(p.row_stat[tile.seq_id * p.stat_sb + head * p.stat_sh + tok0 + key]) *
+                            (float)dob[(int64_t)key * p.d_o.st + d];
         }
-      }
+    }
+    const RowSink<T> dk_sink = make_row_sink<T>(dkb, p.dk.st, L, D), dv_sink = make_row_sink<T>(dvb, p.dv.st, L, D);
+    // Wave-private transposition scratch in the third Q/dO buffer, which nobody touches until the next tile's loop.
+    T* scratch = lds + Lds::kQ + 4 * Lds::kQdoTile + wave * (32 * lds_stride<32>());
+#pragma unroll
+    for (int mt = 0; mt < kMT; mt++) {
+      store_acc_tile_wide<T>(dk_sink, dkacc[mt], p.logit_scale, j0 + 32 * (mt0 + mt), 32 * ct, half, col, lane, scratch);
+      store_acc_tile_wide<T>(dv_sink, dvacc[mt], 1.f, j0 + 32 * (mt0 + mt), 32 * ct, half, col, lane, scratch);
+    }
+      }  // rounds of the tile walk (consumers)
   }
 }
 
 template <typename T, int DH>
-static hipError_t launch_dkv3(const BwdParams& p, int max_tiles, hipStream_t stream) {
+static hipError_t launch_dkv3(const BwdParams& p_in, int max_tiles, hipStream_t stream) {
   const size_t lds_bytes = (size_t)Dkv3Lds<DH>::kElems * sizeof(T);
   // The tile set exceeds the default 64 KB dynamic-LDS cap; the attribute is per device and cheap to set.
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv3_kernel<T, DH>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (e != hipSuccess) return e;
-  const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kDkv3Threads);
+  int dev = 0, cus = 0;
+  if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+  if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+  BwdParams p = p_in;
+  // One workgroup per CU: the same number of workgroups for every head, and with a head count that is a multiple of
+  // 8 the workgroups of a head share an XCD (workgroup ids are dealt round-robin to the 8 XCDs).
+  p.wgs_per_head = cus / p.num_heads > 0 ? cus / p.num_heads : 1;
+  if (p.wgs_per_head > max_tiles) p.wgs_per_head = max_tiles;
+  const dim3 grid((unsigned)(p.wgs_per_head * p.num_heads)), block(kDkv3Threads);
   hipLaunchKernelGGL((bwd_dkv3_kernel<T, DH>), grid, block, lds_bytes, stream, p);
   return hipGetLastError();
 }

@@ -160,6 +160,12 @@ __global__ __launch_bounds__(kThreads, KT == 32 ? 2 : 1) void bwd_dq_kernel(BwdP
   }
 
   T* dqb = (T*)p.dq.ptr + tile.seq_id * p.dq.sb + head * p.dq.sh + tok0 * p.dq.st;
+  if (kFast) {
+    const RowSink<T> sink = make_row_sink<T>(dqb, p.dq.st, L, D);
+#pragma unroll
+    for (int dt = 0; dt < kDTiles; dt++) store_acc_tile<T>(sink, dqacc[dt], p.logit_scale, w_first, 32 * dt, half, col);
+    return;
+  }
 #pragma unroll
   for (int dt = 0; dt < kDTiles; dt++) {
     const int d = 32 * dt + col;

@@ -287,6 +287,60 @@ __device__ __forceinline__ void bwd_tile_math(const f32x16 (&s)[NT], const f32x1
                                      prefix_upper, prefix_out);
 }
 
+// Epilogue stores of the fast path.  An MFMA accumulator tile holds, per lane, one column and 16 rows
+// (8*(r/4) + 4*half + r%4); writing it element by element through 64-bit pointers with a bounds test per row costs
+// ~15 instructions per 2-byte store.  Here the rows of one (head, sequence) are addressed through a raw buffer
+// resource instead: a per-lane byte offset (half-wave row offset + column), a scalar byte offset per register (row
+// * stride), and rows beyond the sequence are dropped by the buffer's range check.  Requires the same conditions as
+// the buffer loads (32-bit offsets within one sequence's rows, head_dim == DH).
+template <typename T>
+struct RowSink {
+  __amdgpu_buffer_rsrc_t rsrc;
+  int stride_bytes;
+};
+template <typename T>
+__device__ __forceinline__ RowSink<T> make_row_sink(T* base, int64_t stride, int rows, int d) {
+  RowSink<T> r;
+  r.stride_bytes = (int)(stride * (int64_t)sizeof(T));
+  const int bytes = rows > 0 ? (rows - 1) * r.stride_bytes + d * (int)sizeof(T) : 0;
+  r.rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
+  return r;
+}
+// acc[r] -> row (row0 + 8*(r/4) + 4*half + r%4), column col0 + (lane % 32), scaled; row0 and col0 wave-uniform.
+template <typename T>
+__device__ __forceinline__ void store_acc_tile(const RowSink<T>& sink, const f32x16& acc, float scale, int row0, int col0,
+                                               int half, int col) {
+  const int voff = 4 * half * sink.stride_bytes + col * (int)sizeof(T);
+  const int sbase = __builtin_amdgcn_readfirstlane(row0 * sink.stride_bytes + col0 * (int)sizeof(T));
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    const T v = (T)(acc[r] * scale);
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, v), sink.rsrc, voff,
+                                          sbase + (8 * (r >> 2) + (r & 3)) * sink.stride_bytes, 0);
+  }
+}
+
+// The same tile through a wave-private LDS scratch of 32 x lds_stride<32>() elements, so that it leaves as two
+// 16-byte stores per lane instead of sixteen 2-byte ones: each lane writes its column's 4-key groups transposed
+// ([column][row] layout, 8 bytes per write), and the transpose read hands every lane 8 consecutive columns of one row.
+template <typename T>
+__device__ __forceinline__ void store_acc_tile_wide(const RowSink<T>& sink, const f32x16& acc, float scale, int row0, int col0,
+                                                    int half, int col, int lane, T* scratch) {
+  constexpr int kStride = lds_stride<32>();
+#pragma unroll
+  for (int g = 0; g < 4; g++) {
+    uint32_t lo = pack2<T>(acc[4 * g] * scale, acc[4 * g + 1] * scale), hi = pack2<T>(acc[4 * g + 2] * scale, acc[4 * g + 3] * scale);
+    *reinterpret_cast<uint64_t*>(scratch + col * kStride + 8 * g + 4 * half) = (uint64_t)lo | ((uint64_t)hi << 32);
+  }
+  const int voff = col * sink.stride_bytes + 8 * half * (int)sizeof(T);
+  const int sbase = __builtin_amdgcn_readfirstlane(row0 * sink.stride_bytes + col0 * (int)sizeof(T));
+#pragma unroll
+  for (int c = 0; c < 2; c++) {
+    const typename Elem<T>::vec8 v = lds_col8<T>(scratch, kStride, 16 * c + 8 * half, 0, lane);   // row `col`, columns 16c+8half..+7
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), sink.rsrc, voff, sbase + 16 * c * (int)sizeof(T), 0);
+  }
+}
+
 // Map the linear workgroup id to (head, tile slot) so that the workgroups of one head land on one XCD
 // (workgroups are dealt round-robin to the 8 XCDs, each with a private L2): K/V of a head are then
 // re-read from that XCD's L2 rather than from HBM.

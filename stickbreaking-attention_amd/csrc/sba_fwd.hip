@@ -164,6 +164,10 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
           ob[(int64_t)row * p.o.st + d] = (T)(oacc[dt][r] + rem_row * (float)vb[(int64_t)row * p.v.st + d]);
       }
     }
+  } else if (kFast) {
+    const RowSink<T> sink = make_row_sink<T>(ob, p.o.st, L, D);
+#pragma unroll
+    for (int dt = 0; dt < kDTiles; dt++) store_acc_tile<T>(sink, oacc[dt], 1.f, w_first, 32 * dt, half, col);
   } else {
 #pragma unroll
     for (int dt = 0; dt < kDTiles; dt++) {

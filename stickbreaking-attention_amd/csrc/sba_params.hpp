@@ -71,6 +71,7 @@ struct BwdParams {
   int32_t add_rem;
   const float* row_stat;       // log2(rem), fp32 [batch][head][token]
   int64_t stat_sb, stat_sh;
+  int32_t wgs_per_head;        // persistent dK/dV workgroups per head
   float* drem_eff;             // workspace, indexed like row_stat: the gradient of rem per row in fp32 (d_rem, plus
                                // d_o . v when add_rem), written by the dQ kernel and read by the dK/dV kernel
 };
