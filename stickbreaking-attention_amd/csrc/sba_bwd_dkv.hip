@@ -375,6 +375,45 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
     }  // rounds of the tile walk (producers)
   } else {
     if (slot_of(0) < n_tiles) stage_first(next_tile);
+    // Output blocks of this consumer wave.  head_dim 128: both 32-key row tiles x columns 32*wave .. +31;
+    // head_dim 64: row tile wave/2 x columns 32*(wave%2) .. +31.
+    constexpr int kMT = DH == 128 ? 2 : 1;
+    const int mt0 = DH == 128 ? 0 : wave >> 1, ct = DH == 128 ? wave : wave & 1;
+    f32x16 dkacc[kMT], dvacc[kMT];
+    // The results of a tile are stored during the first step of the NEXT tile, when the consumers have nothing to
+    // contract yet (and after the last tile): acc[mt][r] is key origin + 32*(mt0 + mt) + 8*(r/4) + 4*half + r%4,
+    // column 32*ct + col.
+    bool pending = false;
+    Tile done_tile = next_tile;
+    auto store_results = [&](const Tile& tl) {
+      const int tl_len = tl.seq_len, tl_j0 = tl.origin;
+      const int64_t tl_tok0 = tl.seq_start;
+      T* dkb = (T*)p.dk.ptr + tl.seq_id * p.dk.sb + head * p.dk.sh + tl_tok0 * p.dk.st;
+      T* dvb = (T*)p.dv.ptr + tl.seq_id * p.dv.sb + head * p.dv.sh + tl_tok0 * p.dv.st;
+      if (p.add_rem) {
+        // the remainder term o += rem * v contributes rem_j * d_o_j to dv_j
+        const T* dob = (const T*)p.d_o.ptr + tl.seq_id * p.d_o.sb + head * p.d_o.sh + tl_tok0 * p.d_o.st;
+        const int d = 32 * ct + col;
+#pragma unroll
+        for (int mt = 0; mt < kMT; mt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int key = tl_j0 + 32 * (mt0 + mt) + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (key < tl_len)
+              dvacc[mt][r] += fast_exp2(p.row_stat[tl.seq_id * p.stat_sb + head * p.stat_sh + tl_tok0 + key]) *
+                              (float)dob[(int64_t)key * p.d_o.st + d];
+          }
+      }
+      const RowSink<T> dk_sink = make_row_sink<T>(dkb, p.dk.st, tl_len, DH), dv_sink = make_row_sink<T>(dvb, p.dv.st, tl_len, DH);
+      // Wave-private transposition scratch in the third Q/dO buffer: free during a tile's first step and after the
+      // last one.
+      T* scratch = lds + Lds::kQ + 4 * Lds::kQdoTile + wave * (32 * lds_stride<32>());
+#pragma unroll
+      for (int mt = 0; mt < kMT; mt++) {
+        store_acc_tile_wide<T>(dk_sink, dkacc[mt], p.logit_scale, tl_j0 + 32 * (mt0 + mt), 32 * ct, half, col, lane, scratch);
+        store_acc_tile_wide<T>(dv_sink, dvacc[mt], 1.f, tl_j0 + 32 * (mt0 + mt), 32 * ct, half, col, lane, scratch);
+      }
+    };
   for (int round = 0; wph * round < n_tiles; ++round) {
   const int slot = slot_of(round);
   if (slot >= n_tiles) break;                                // only in the last, partial round
@@ -384,22 +423,11 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
   if (have_next) next_tile = p.k_tiles[next_slot];
   const int L = tile.seq_len, j0 = tile.origin, ac = p.attend_current, D = DH;
   const int64_t tok0 = tile.seq_start;
-  const int jt = j0 / kBlockK;
 
   const int first_row = j0 + 1 - ac;                         // first row that sees key j0
-  const int n_qt = (L + kBlockQ - 1) / kBlockQ;
   const int row_begin = first_row < L ? (first_row / kDkvRows) * kDkvRows : L;
   const int n_steps = (L - row_begin + kDkvRows - 1) / kDkvRows;
 
-    // Output blocks of this consumer wave.  head_dim 128: both 32-key row tiles x columns 32*wave .. +31;
-    // head_dim 64: row tile wave/2 x columns 32*(wave%2) .. +31.
-    constexpr int kMT = DH == 128 ? 2 : 1;
-    const int mt0 = DH == 128 ? 0 : wave >> 1, ct = DH == 128 ? wave : wave & 1;
-    f32x16 dkacc[kMT], dvacc[kMT];
-#pragma unroll
-    for (int b = 0; b < kMT; b++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) { dkacc[b][r] = 0.f; dvacc[b][r] = 0.f; }
     // The consumers also move the query tiles global -> registers -> LDS (they have the issue slots to spare):
     // tile t+1 is written at the top of step t from registers loaded during step t-1, then tile t+2 is requested;
     // the barrier that ends a step is the only point that waits for those loads.
@@ -415,7 +443,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
       }
     }
     __syncthreads();
-    for (int t = 0; t <= n_steps; ++t) {
+    auto stage_step = [&](int t) {          // rows of step t+1 into LDS, rows of step t+2 requested
       if (t + 1 < n_steps) {
         T* nq_lds = lds + Lds::kQ + ((t + 1) % 3) * 2 * Lds::kQdoTile;
         cq.store(nq_lds);
@@ -426,7 +454,18 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
           cdo.load(dosrc, qn);
         }
       }
-      if (t >= 1) {
+    };
+    // Step 0: nothing to contract yet, so the previous tile's results leave now.
+    stage_step(0);
+    if (pending) store_results(done_tile);
+#pragma unroll
+    for (int b = 0; b < kMT; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) { dkacc[b][r] = 0.f; dvacc[b][r] = 0.f; }
+    __syncthreads();
+    for (int t = 1; t <= n_steps; ++t) {
+      stage_step(t);
+      {
         const int u = t - 1;
         const T* q_lds = lds + Lds::kQ + (u % 3) * 2 * Lds::kQdoTile;
         const T* do_lds = q_lds + Lds::kQdoTile;
@@ -450,31 +489,10 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
       __syncthreads();
     }
     if (have_next) stage_first(next_tile);
-    // acc[mt][r]: key j0 + 32*(mt0 + mt) + 8*(r/4) + 4*half + r%4, column 32*ct + col.
-    T* dkb = (T*)p.dk.ptr + tile.seq_id * p.dk.sb + head * p.dk.sh + tok0 * p.dk.st;
-    T* dvb = (T*)p.dv.ptr + tile.seq_id * p.dv.sb + head * p.dv.sh + tok0 * p.dv.st;
-    const int d = 32 * ct + col;
-    if (p.add_rem) {
-      // the remainder term o += rem * v contributes rem_j * d_o_j to dv_j
-#pragma unroll
-      for (int mt = 0; mt < kMT; mt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int key = j0 + 32 * (mt0 + mt) + 8 * (r >> 2) + 4 * half + (r & 3);
-          if (key < L)
-            dvacc[mt][r] += fast_exp2(p.row_stat[tile.seq_id * p.stat_sb + head * p.stat_sh + tok0 + key]) *
-                            (float)dob[(int64_t)key * p.d_o.st + d];
-        }
-    }
-    const RowSink<T> dk_sink = make_row_sink<T>(dkb, p.dk.st, L, D), dv_sink = make_row_sink<T>(dvb, p.dv.st, L, D);
-    // Wave-private transposition scratch in the third Q/dO buffer, which nobody touches until the next tile's loop.
-    T* scratch = lds + Lds::kQ + 4 * Lds::kQdoTile + wave * (32 * lds_stride<32>());
-#pragma unroll
-    for (int mt = 0; mt < kMT; mt++) {
-      store_acc_tile_wide<T>(dk_sink, dkacc[mt], p.logit_scale, j0 + 32 * (mt0 + mt), 32 * ct, half, col, lane, scratch);
-      store_acc_tile_wide<T>(dv_sink, dvacc[mt], 1.f, j0 + 32 * (mt0 + mt), 32 * ct, half, col, lane, scratch);
-    }
+    pending = true;
+    done_tile = tile;
       }  // rounds of the tile walk (consumers)
+    if (pending) store_results(done_tile);
   }
 }
 
