@@ -23,7 +23,7 @@ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 struct Layout {
   int64_t max_q_tiles, max_k_tiles, carry_slots_per_head;
-  size_t off_counts, off_q_tiles, off_k_tiles, off_carry_base, off_prefix, off_drem;
+  size_t off_counts, off_q_tiles, off_k_tiles, off_carry_base, off_prefix, off_drem, off_queue;
   size_t fwd_bytes, bwd_bytes, carry_bytes;
 };
 
@@ -56,6 +56,7 @@ int plan(const SbaArgs* a, Layout* out) {
   L.off_prefix = off;      off += L.carry_bytes;
   // d_rem + d_o . v per row (fp32), used when the remainder term is fused
   L.off_drem = off;        off = align_up(off + (size_t)a->num_heads * (size_t)T * (fixed ? (size_t)B : 1) * sizeof(float), 256);
+  L.off_queue = off;       off = align_up(off + (size_t)a->num_heads * sizeof(int32_t), 256);      // per-head tile cursors
   L.bwd_bytes = off;
   *out = L;
   return SBA_OK;
@@ -96,6 +97,8 @@ int run_sched(const SbaArgs* a, const Layout& L, bool want_key_tiles, bool want_
   sp.k_tiles = (sba::Tile*)(ws + L.off_k_tiles);
   sp.counts = (int32_t*)(ws + L.off_counts);
   sp.carry_base = (int64_t*)(ws + L.off_carry_base);
+  sp.head_queue = (int32_t*)(ws + L.off_queue);
+  sp.num_heads = a->num_heads;
   return sba::launch_sched(sp, stream) == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
 }
 
@@ -221,6 +224,7 @@ int sba_bwd(const SbaArgs* a) {
   p.stat_sb = fixed ? (int64_t)a->num_heads * a->total_tokens : 0;
   p.stat_sh = a->total_tokens;
   p.drem_eff = (float*)(ws + L.off_drem);
+  p.head_queue = (int32_t*)(ws + L.off_queue);
   const int64_t max_rows = (a->max_seqlen > 0 && a->max_seqlen < a->total_tokens) ? a->max_seqlen : a->total_tokens;
   bool v16 = (a->head_dim % (16 / (int)es)) == 0;
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})

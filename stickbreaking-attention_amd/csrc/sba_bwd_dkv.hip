@@ -226,8 +226,9 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
   const bool producer = threadIdx.x < 256;
   const int half = lane >> 5, col = lane & 31;
   const int ac = p.attend_current;
-  // The `wph` workgroups of a head take the tiles of that head's list (heaviest first) in rounds of wph, in
-  // alternating order, so that every workgroup gets the same share of heavy and light tiles.
+  // The `wph` workgroups of a head start with the head's first wph tiles (the list is heaviest first) and then take
+  // the next tile from a per-head cursor whenever they finish one, so the load balances itself.  The cursor is read
+  // a tile ahead: thread 0 takes the slot after next before a tile's start-up barrier and publishes it through LDS.
   const int wph = p.wgs_per_head;
   int head, w;
   if ((p.num_heads & 7) == 0) {
@@ -238,14 +239,14 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
     head = blockIdx.x % p.num_heads;
     w = blockIdx.x / p.num_heads;
   }
-  auto slot_of = [&](int round) { return wph * round + ((round & 1) ? wph - 1 - w : w); };
+  int* next_slot_lds = reinterpret_cast<int*>(lds_raw + (size_t)Lds::kElems * sizeof(T));
   auto first_row_block = [&](const Tile& tl) {               // first 64-row step that sees the tile's first key
     const int first_row = tl.origin + 1 - ac;
     return first_row < tl.seq_len ? (first_row / kDkvRows) * kDkvRows : tl.seq_len;
   };
   // The tile record of the next round is fetched a round ahead; the consumers also request the first query rows
   // of the next tile before they store the results of the current one.
-  Tile next_tile = p.k_tiles[slot_of(0) < n_tiles ? slot_of(0) : 0];
+  Tile next_tile = p.k_tiles[w < n_tiles ? w : 0];
   TileCopy<T, DH, kDkvRows, true> cq, cdo;                   // staging registers (consumer waves)
   auto stage_first = [&](const Tile& tl) {
     const T* qb = (const T*)p.q.ptr + tl.seq_id * p.q.sb + head * p.q.sh + (int64_t)tl.seq_start * p.q.st;
@@ -272,14 +273,10 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
   // Each role runs its own walk over the same rounds (same tiles, same number of barriers), so that what one role
   // carries from tile to tile does not occupy registers in the other role's code.
   if (producer) {
-    if (slot_of(0) < n_tiles) load_kv(next_tile);
-  for (int round = 0; wph * round < n_tiles; ++round) {
-  const int slot = slot_of(round);
-  if (slot >= n_tiles) break;                                // only in the last, partial round
+    if (w < n_tiles) load_kv(next_tile);
+  for (int slot = w; slot < n_tiles;) {
   const Tile tile = next_tile;
-  const int next_slot = slot_of(round + 1);
-  const bool have_next = next_slot < n_tiles;
-  if (have_next) next_tile = p.k_tiles[next_slot];
+  if (threadIdx.x == 0) *next_slot_lds = wph + atomicAdd(p.head_queue + head, 1);
   const int L = tile.seq_len, j0 = tile.origin, ac = p.attend_current, D = DH;
   const int64_t tok0 = tile.seq_start;
   const int jt = j0 / kBlockK;
@@ -315,7 +312,12 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
     };
     if (n_steps > 0) fetch_row_scalars(row_begin);
     __syncthreads();
-    if (have_next) load_kv(next_tile);
+    slot = *next_slot_lds;                                   // the tile after this one
+    const bool have_next = slot < n_tiles;
+    if (have_next) {
+      next_tile = p.k_tiles[slot];
+      load_kv(next_tile);
+    }
     for (int t = 0; t <= n_steps; ++t) {
       if (t < n_steps) {
         const int q0 = row_begin + t * kDkvRows;
@@ -374,7 +376,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
     }
     }  // rounds of the tile walk (producers)
   } else {
-    if (slot_of(0) < n_tiles) stage_first(next_tile);
+    if (w < n_tiles) stage_first(next_tile);
     // Output blocks of this consumer wave.  head_dim 128: both 32-key row tiles x columns 32*wave .. +31;
     // head_dim 64: row tile wave/2 x columns 32*(wave%2) .. +31.
     constexpr int kMT = DH == 128 ? 2 : 1;
@@ -414,13 +416,8 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
         store_acc_tile_wide<T>(dv_sink, dvacc[mt], 1.f, tl_j0 + 32 * (mt0 + mt), 32 * ct, half, col, lane, scratch);
       }
     };
-  for (int round = 0; wph * round < n_tiles; ++round) {
-  const int slot = slot_of(round);
-  if (slot >= n_tiles) break;                                // only in the last, partial round
+  for (int slot = w; slot < n_tiles;) {
   const Tile tile = next_tile;
-  const int next_slot = slot_of(round + 1);
-  const bool have_next = next_slot < n_tiles;
-  if (have_next) next_tile = p.k_tiles[next_slot];
   const int L = tile.seq_len, j0 = tile.origin, ac = p.attend_current, D = DH;
   const int64_t tok0 = tile.seq_start;
 
@@ -443,6 +440,9 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
       }
     }
     __syncthreads();
+    slot = *next_slot_lds;                                   // the tile after this one
+    const bool have_next = slot < n_tiles;
+    if (have_next) next_tile = p.k_tiles[slot];
     auto stage_step = [&](int t) {          // rows of step t+1 into LDS, rows of step t+2 requested
       if (t + 1 < n_steps) {
         T* nq_lds = lds + Lds::kQ + ((t + 1) % 3) * 2 * Lds::kQdoTile;
@@ -498,7 +498,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
 
 template <typename T, int DH>
 static hipError_t launch_dkv3(const BwdParams& p_in, int max_tiles, hipStream_t stream) {
-  const size_t lds_bytes = (size_t)Dkv3Lds<DH>::kElems * sizeof(T);
+  const size_t lds_bytes = (size_t)Dkv3Lds<DH>::kElems * sizeof(T) + 256;      // + the published queue slot
   // The tile set exceeds the default 64 KB dynamic-LDS cap; the attribute is per device and cheap to set.
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv3_kernel<T, DH>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);

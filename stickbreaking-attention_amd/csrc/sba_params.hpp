@@ -33,6 +33,8 @@ struct SchedParams {
   Tile* k_tiles;           // key tiles (kBlockK keys), heaviest first
   int32_t* counts;         // [0] = number of query tiles, [1] = number of key tiles
   int64_t* carry_base;     // per sequence: first carry slot of the sequence (per head)
+  int32_t* head_queue;     // backward: per-head cursor into the key-tile list, reset to 0 here
+  int32_t num_heads;
 };
 
 struct FwdParams {
@@ -72,6 +74,7 @@ struct BwdParams {
   const float* row_stat;       // log2(rem), fp32 [batch][head][token]
   int64_t stat_sb, stat_sh;
   int32_t wgs_per_head;        // persistent dK/dV workgroups per head
+  int32_t* head_queue;         // per head: next key tile not yet taken (beyond the first wgs_per_head), zero at launch
   float* drem_eff;             // workspace, indexed like row_stat: the gradient of rem per row in fp32 (d_rem, plus
                                // d_o . v when add_rem), written by the dQ kernel and read by the dK/dV kernel
 };

@@ -114,6 +114,8 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
     p.counts[0] = qbins[0];
     p.counts[1] = p.want_key_tiles ? kbins[0] : 0;
   }
+  if (p.want_key_tiles)
+    for (int h = threadIdx.x; h < p.num_heads; h += kSchedThreads) p.head_queue[h] = 0;
 
   // Carry layout: exclusive prefix sum of carry_slots(M_s) over sequences (block-wide, chunked).
   if (p.want_carry_base) {
