@@ -81,7 +81,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
   const int n_qt = (L + kBlockQ - 1) / kBlockQ;
   const int qt_begin = first_row < L ? first_row / kBlockQ : n_qt;    // == jt / 2 whenever any row sees the tile
   // product above the tile = above its upper 32-key sub-tile; prefix below the tile = below its lower sub-tile
-  const int64_t seq0 = (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] - (int64_t)kBlockQ * (jt >> 1);
+  const int64_t seq0 = (int64_t)head * p.carry_head_stride + tile.carry_base - (int64_t)kBlockQ * (jt >> 1);
   const float* carry = p.carry + seq0 + carry_offset(2 * jt + 1, n_qt);      // + row
   const float* prefix = p.prefix + seq0 + carry_offset(2 * jt, n_qt);
 
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
     const T* kb = (const T*)p.k.ptr + tile.seq_id * p.k.sb + head * p.k.sh + tok0 * p.k.st;
     const T* vb = (const T*)p.v.ptr + tile.seq_id * p.v.sb + head * p.v.sh + tok0 * p.v.st;
     const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
-    const int64_t slot0 = (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] +
+    const int64_t slot0 = (int64_t)head * p.carry_head_stride + tile.carry_base +
                           carry_offset(2 * jt + group, n_qt) - (int64_t)kBlockQ * (jt >> 1);      // + row
     const float* carry = p.carry + slot0;
     const float* prefix = p.prefix + slot0;

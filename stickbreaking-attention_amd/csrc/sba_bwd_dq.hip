@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kThreads, KT == 32 ? 2 : 1) void bwd_dq_kernel(BwdP
   const int n_kt = last_key < 0 ? 0 : last_key / KT + 1;
   const int w_first = q0 + wave * 32, w_last = w_first + 31;
   const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
-  const int64_t slot0 = (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id];
+  const int64_t slot0 = (int64_t)head * p.carry_head_stride + tile.carry_base;
   const float* carry = p.carry + slot0;
   float* prefix_out = p.prefix + slot0;
 

@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kThreads) void fwd_f32_kernel(FwdParams p) {
   const float* vb = (const float*)p.v.ptr + tile.seq_id * p.v.sb + head * p.v.sh + tok0 * p.v.st;
   float* ob = (float*)p.o.ptr + tile.seq_id * p.o.sb + head * p.o.sh + tok0 * p.o.st;
   const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
-  float* carry = p.carry ? p.carry + (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] : nullptr;
+  float* carry = p.carry ? p.carry + (int64_t)head * p.carry_head_stride + tile.carry_base : nullptr;
 
   for (int r = 0; r < kF32RowsPerWave; r++) {
     const int i = row_base + r;
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_kernel(BwdParams p) {
   float* dkb = (float*)p.dk.ptr + tile.seq_id * p.dk.sb + head * p.dk.sh + tok0 * p.dk.st;
   float* dvb = (float*)p.dv.ptr + tile.seq_id * p.dv.sb + head * p.dv.sh + tok0 * p.dv.st;
   const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
-  const float* carry = p.carry + (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id];
+  const float* carry = p.carry + (int64_t)head * p.carry_head_stride + tile.carry_base;
 
   const int wg_last_key = min(wg_row0 + kF32Rows, L) - 2 + ac;
   const int n_steps = (wg_last_key < 0 || wg_row0 >= L) ? 0 : wg_last_key / kF32Keys + 1;

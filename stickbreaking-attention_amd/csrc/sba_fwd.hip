@@ -57,7 +57,7 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
     for (int r = 0; r < 16; r++) oacc[dt][r] = 0.f;
   float prod = 1.f;    // prod over the keys already swept of (1 - sigma): both half-waves hold the same value
   const int64_t n_qt = (L + kBlockQ - 1) / kBlockQ;
-  float* carry = p.carry ? p.carry + (int64_t)head * p.carry_head_stride + p.carry_base[tile.seq_id] : nullptr;
+  float* carry = p.carry ? p.carry + (int64_t)head * p.carry_head_stride + tile.carry_base : nullptr;
 
   const RowSource<T> ksrc = make_row_source<T, kFast>(kb, p.k.st, L, D), vsrc = make_row_source<T, kFast>(vb, p.v.st, L, D);
   TileCopy<T, DH, KT, kFast> ck, cv;

@@ -19,6 +19,7 @@ struct Tile {
   int32_t seq_len;
   int32_t origin;      // first query row (query tiles) or first key (key tiles), relative to the sequence
   int32_t seq_id;      // sequence index; selects the batch stride in fixed-length mode
+  int64_t carry_base;  // first carry slot of the sequence within a head's plane (0 when no carries are laid out)
 };
 
 struct SchedParams {

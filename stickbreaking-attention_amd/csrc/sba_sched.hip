@@ -84,39 +84,6 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
   descending_offsets(qbins, scratch);
   if (p.want_key_tiles) descending_offsets(kbins, scratch);
 
-  // Pass 2: each sequence takes a contiguous range of slots in its class; one wave per sequence.
-  for (int s = wave; s < p.num_seqs; s += nwaves) {
-    int start, len;
-    seq_bounds(p, s, &start, &len);
-    const int nq = (len + kBlockQ - 1) / kBlockQ, nk = (len + kBlockK - 1) / kBlockK;
-    const int cls = min(nq, kBins - 1);
-    int qbase = 0, kbase = 0;
-    if (lane == 0) {
-      if (nq) qbase = atomicAdd(&qbins[cls], nq);
-      if (nk && p.want_key_tiles) kbase = atomicAdd(&kbins[cls], nk);
-    }
-    qbase = __shfl(qbase, 0);
-    kbase = __shfl(kbase, 0);
-    for (int t = lane; t < nq; t += 64) {        // heaviest query tile (the last one) first
-      Tile d; d.seq_start = start; d.seq_len = len; d.origin = (nq - 1 - t) * kBlockQ; d.seq_id = s;
-      p.q_tiles[qbase + t] = d;
-    }
-    if (p.want_key_tiles) {
-      for (int t = lane; t < nk; t += 64) {      // heaviest key tile (the first one) first
-        Tile d; d.seq_start = start; d.seq_len = len; d.origin = t * kBlockK; d.seq_id = s;
-        p.k_tiles[kbase + t] = d;
-      }
-    }
-  }
-  __syncthreads();
-  // After the scatter, the lightest bin (work 0) ends at the total count.
-  if (threadIdx.x == 0) {
-    p.counts[0] = qbins[0];
-    p.counts[1] = p.want_key_tiles ? kbins[0] : 0;
-  }
-  if (p.want_key_tiles)
-    for (int h = threadIdx.x; h < p.num_heads; h += kSchedThreads) p.head_queue[h] = 0;
-
   // Carry layout: exclusive prefix sum of carry_slots(M_s) over sequences (block-wide, chunked).
   if (p.want_carry_base) {
     for (int s0 = 0; s0 < p.num_seqs; s0 += kSchedThreads) {
@@ -142,6 +109,42 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
       __syncthreads();
     }
   }
+  __syncthreads();
+
+  // Pass 2: each sequence takes a contiguous range of slots in its class; one wave per sequence.
+  for (int s = wave; s < p.num_seqs; s += nwaves) {
+    int start, len;
+    seq_bounds(p, s, &start, &len);
+    const int nq = (len + kBlockQ - 1) / kBlockQ, nk = (len + kBlockK - 1) / kBlockK;
+    const int cls = min(nq, kBins - 1);
+    int qbase = 0, kbase = 0;
+    if (lane == 0) {
+      if (nq) qbase = atomicAdd(&qbins[cls], nq);
+      if (nk && p.want_key_tiles) kbase = atomicAdd(&kbins[cls], nk);
+    }
+    qbase = __shfl(qbase, 0);
+    kbase = __shfl(kbase, 0);
+    const int64_t cbase = p.want_carry_base ? p.carry_base[s] : 0;      // written above by this workgroup
+    for (int t = lane; t < nq; t += 64) {        // heaviest query tile (the last one) first
+      Tile d; d.seq_start = start; d.seq_len = len; d.origin = (nq - 1 - t) * kBlockQ; d.seq_id = s; d.carry_base = cbase;
+      p.q_tiles[qbase + t] = d;
+    }
+    if (p.want_key_tiles) {
+      for (int t = lane; t < nk; t += 64) {      // heaviest key tile (the first one) first
+        Tile d; d.seq_start = start; d.seq_len = len; d.origin = t * kBlockK; d.seq_id = s; d.carry_base = cbase;
+        p.k_tiles[kbase + t] = d;
+      }
+    }
+  }
+  __syncthreads();
+  // After the scatter, the lightest bin (work 0) ends at the total count.
+  if (threadIdx.x == 0) {
+    p.counts[0] = qbins[0];
+    p.counts[1] = p.want_key_tiles ? kbins[0] : 0;
+  }
+  if (p.want_key_tiles)
+    for (int h = threadIdx.x; h < p.num_heads; h += kSchedThreads) p.head_queue[h] = 0;
+
 }
 
 hipError_t launch_sched(const SchedParams& p, hipStream_t stream) {
