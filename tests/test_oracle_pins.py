@@ -220,7 +220,7 @@ def test_mask_fill_quirks_fp32():
 
 
 def test_fp32_dense_vs_fp64_stream_config1():
-    # BASELINE config 1 shape: fp32, H=4, D=64, lengths [128, 256, 64]; fp32 dense restatement stays within 1e-5 of fp64
+    # configuration C1 shape: fp32, H=4, D=64, lengths [128, 256, 64]; fp32 dense restatement stays within 1e-5 of fp64
     g = torch.Generator().manual_seed(0)
     H, D, cu = 4, 64, [128, 384, 448]
     q, k, v, do = (torch.randn(H, 448, D, generator=g) for _ in range(4))
