@@ -1,7 +1,7 @@
 // Backward, kernel 1 of 2: dQ, plus the per-(row, key tile) prefix sums that make the dK/dV kernel lock-free.
 //
 // One workgroup per tile of 128 query rows (wave w owns rows 32w..32w+31, lane l owns query l%32), key tiles
-// of 64 swept FORWARDS from key 0 to the diagonal.  With g_ij = A_ij (dO_i.v_j - drem_i) the logit gradient is
+// of KT keys (32 on the fast paths, else 64) swept FORWARDS from key 0 to the diagonal.  With g_ij = A_ij (dO_i.v_j - drem_i) the logit gradient is
 //     dz_ij = g_ij - sigma_ij * C_ij,     C_ij = sum_{j' <= j} g_ij'        (sb_varlen_bwd.py:438-447)
 // so C is a running prefix sum in this direction and needs no anchor.  (sigma does not decay with distance, so
 // any constant error in C would be multiplied into every key of the row; C has to be built from exactly the g

@@ -75,13 +75,6 @@ __device__ __forceinline__ float fast_min(float a, float b) {
   return r;
 }
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the vector-memory counter, which
-// would stall on global loads that were deliberately left in flight across the barrier (register prefetch of
-// the next tile).  Nothing here communicates through global memory inside a kernel.
-__device__ __forceinline__ void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
 // Value held by the other half-wave (lane ^ 32).
 __device__ __forceinline__ float other_half(float x, int half) {
   uint32_t u = __builtin_bit_cast(uint32_t, x);
@@ -213,7 +206,6 @@ __device__ __forceinline__ u32x4 load_row8(const T* row, int d0, int d_valid, bo
   return v;
 }
 
-constexpr float kExpClamp = 100.0f;   // 2^100 and 2^-100 are finite; sigma(z) is 1 - 2^-100 there
 
 // Element-wise backward math of one 64-key tile for the 32 keys this lane owns (see the conventions above).
 //   s, dp     : S^T = K Q^T and dP^T = V dO^T accumulators (row tile mt, register r  <->  key 32*half + 16*mt + r)

@@ -1,13 +1,14 @@
 // Forward stick-breaking attention for gfx950.
 //
 // One workgroup = one tile of 128 query rows of one (head, sequence); wave w owns rows 32w..32w+31, lane l
-// owns query l%32.  Key tiles of 64 keys are swept in REVERSE from the causal diagonal (the order in which
-// the stick is broken: stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:155-165), so the running product
+// owns query l%32.  Key tiles of KT keys (32 on the head_dim 128 fast path, else 64) are swept in REVERSE from the
+// causal diagonal (the order in which the stick is broken:
+// stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:155-165), so the running product
 // prod_{j<k<i} (1 - sigma(z_ik)) is carried forward in registers and never has to be divided out.
 //
 // Per element, in linear space (base-2 exponentials, as sb_varlen_fwd.py:296 and softplus.py:8-12 do):
-//     e = 2^x, x = z log2(e)          1 - sigma = 1/(1+e)          sigma = e/(1+e)
-//     A_ij = e_ij * prod_{j<=k<i} 1/(1+e_ik)
+//     e = 2^x, x = z log2(e)          1 - sigma = 1/(1+e)          R_ij = prod_{j<=k<i} 1/(1+e_ik)
+//     A_ij = sigma_ij R_i,j+1 = R_i,j+1 - R_ij
 // which needs two transcendentals (v_exp_f32, v_rcp_f32) where the log-space form
 // log A = x - softplus2(x) + cumsum(-softplus2) needs three.  The product can only underflow where A itself is
 // below 2^-126, and row_stat = log2(prod) is taken once per row at the end.
