@@ -9,6 +9,7 @@ hipError_t launch_sched(const SchedParams& p, hipStream_t stream);
 hipError_t launch_fwd(const FwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
 hipError_t launch_bwd_dq(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
 hipError_t launch_bwd_dkv(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
+int dkv_key_tile(const BwdParams& p);
 hipError_t launch_fwd_f32(const FwdParams& p, int max_tiles, hipStream_t stream);
 hipError_t launch_bwd_f32(const BwdParams& p, int batches, int64_t tokens, int max_q_tiles, hipStream_t stream);
 }  // namespace sba
@@ -82,7 +83,7 @@ int check_tensor(const SbaTensor& t, bool required, bool fixed) {
 sba::TensorRef ref(const SbaTensor& t, bool fixed) { return sba::TensorRef{t.ptr, fixed ? t.stride_batch : 0, t.stride_head, t.stride_token}; }
 sba::VectorRef vref(const SbaVector& t, bool fixed) { return sba::VectorRef{t.ptr, fixed ? t.stride_batch : 0, t.stride_head, t.stride_token}; }
 
-int run_sched(const SbaArgs* a, const Layout& L, bool want_key_tiles, bool want_carry_base, hipStream_t stream) {
+int run_sched(const SbaArgs* a, const Layout& L, bool want_key_tiles, bool want_carry_base, int key_tile, hipStream_t stream) {
   char* ws = (char*)a->workspace;
   sba::SchedParams sp{};
   sp.cu = a->cu_seqlens;
@@ -99,6 +100,7 @@ int run_sched(const SbaArgs* a, const Layout& L, bool want_key_tiles, bool want_
   sp.carry_base = (int64_t*)(ws + L.off_carry_base);
   sp.head_queue = (int32_t*)(ws + L.off_queue);
   sp.num_heads = a->num_heads;
+  sp.key_tile = key_tile;
   return sba::launch_sched(sp, stream) == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
 }
 
@@ -149,7 +151,7 @@ int sba_fwd(const SbaArgs* a) {
     if (t->ptr && ((uintptr_t)t->ptr % es)) return SBA_ERR_ALIGN;
   if (!a->workspace || ((uintptr_t)a->workspace & 255) || a->workspace_bytes < L.fwd_bytes) return SBA_ERR_WORKSPACE;
   hipStream_t stream = (hipStream_t)a->stream;
-  if ((st = run_sched(a, L, false, a->carry != nullptr, stream)) != SBA_OK) return st;
+  if ((st = run_sched(a, L, false, a->carry != nullptr, kBlockK, stream)) != SBA_OK) return st;
 
   char* ws = (char*)a->workspace;
   sba::FwdParams p{};
@@ -199,7 +201,6 @@ int sba_bwd(const SbaArgs* a) {
     if (t->ptr && ((uintptr_t)t->ptr % es)) return SBA_ERR_ALIGN;
   if (!a->workspace || ((uintptr_t)a->workspace & 255) || a->workspace_bytes < L.bwd_bytes) return SBA_ERR_WORKSPACE;
   hipStream_t stream = (hipStream_t)a->stream;
-  if ((st = run_sched(a, L, true, true, stream)) != SBA_OK) return st;
 
   char* ws = (char*)a->workspace;
   sba::BwdParams p{};
@@ -230,6 +231,9 @@ int sba_bwd(const SbaArgs* a) {
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
     if (t->ptr) v16 = v16 && vec16(*t, es, fixed, max_rows);
   p.vec_ok = v16 ? 1 : 0;
+  // The key-tile list is built for the dK/dV kernel that will run (the fp32 kernels do not use it).
+  const int key_tile = a->dtype == SBA_F32 ? kBlockK : sba::dkv_key_tile(p);
+  if ((st = run_sched(a, L, true, true, key_tile, stream)) != SBA_OK) return st;
   hipEvent_t* ev = (hipEvent_t*)a->trace_events;
   if (ev && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;
   if (a->dtype == SBA_F32) {

@@ -14,6 +14,8 @@
 #include "sba_device.hpp"
 #include "sba_params.hpp"
 
+#include <type_traits>
+
 namespace sba {
 
 template <int DH> struct DkvLds {
@@ -516,6 +518,381 @@ static hipError_t launch_dkv3(const BwdParams& p_in, int max_tiles, hipStream_t 
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Software-pipelined producer / consumer kernel: 128-key tiles swept by steps of 32 query rows.
+//
+// In the kernel above a producer wave's step is one serial chain -- wait for the B operands from LDS, 16 MFMAs,
+// the element-wise math, the LDS writes, the barrier -- and with one producer per SIMD nothing else on that SIMD
+// has vector-ALU work to fill the waits.  Here the producer issues the MFMAs of step t+1 (S^T and dP^T of the
+// next 32 rows) inside the same straight-line block as the math of step t, so the matrix pipe runs under the
+// vector ALU and the LDS latency is off the chain.  That needs the query rows in LDS one step earlier (4 stages
+// of {Q, dO} instead of 3), which fits because a step is 32 rows; the tile is 128 keys so that a step still has
+// one 32x32 block per producer wave.  Wave g of the producers owns the 32-key sub-tile g (K/V operands stationary
+// in registers) and all four sweep the same rows; consumer wave (mp, cp) owns keys 64*mp..+63 x columns
+// (DH/2)*cp..+DH/2-1 of dK and dV, which halves the LDS operand reads per MFMA of the narrower layout.
+//
+// Rows of step r (relative to the tile's first step): requested from global memory at step r-4, written to LDS
+// stage r%4 at step r-2, read by the producers at step r-1 (MFMAs) and by the consumers at step r+1; P/dZ of
+// step r are written at step r into buffer r%2 and contracted at step r+1.
+constexpr int kDkv4Keys = 128;
+constexpr int kDkv4Rows = 32;
+constexpr int kDkv4Threads = 512;
+template <int DH> struct Dkv4Lds {
+  static constexpr int kRowStride = lds_stride<DH>();
+  static constexpr int kPStride = lds_stride<kDkv4Keys>();
+  static constexpr int kQdoTile = kDkv4Rows * kRowStride;    // one Q (or dO) tile
+  static constexpr int kPTile = kDkv4Rows * kPStride;        // one P (or dZ) tile
+  static constexpr int kQ = 0;                               // 4 stages of {Q, dO}
+  static constexpr int kP = 8 * kQdoTile;                    // 2 buffers of {P, dZ}
+  static constexpr int kScratch = kP + 4 * kPTile;           // one transposition scratch per consumer wave
+  static constexpr int kElems = kScratch + 4 * 32 * lds_stride<32>();
+};
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the vector-memory counter, which
+// would stall on the global loads that are deliberately left in flight across the barrier (staging registers,
+// next tile's operands).  Nothing in this kernel communicates through global memory.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <typename T, int DH>
+__global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
+  typedef typename Elem<T>::vec8 vec8;
+  typedef Dkv4Lds<DH> Lds;
+  constexpr int kRowStride = Lds::kRowStride, kPStride = Lds::kPStride;
+  constexpr int kSteps = DH / 16;
+  constexpr int kRows = kDkv4Rows;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+
+  // Persistent workgroups, one per CU, each walking the key-tile list of one head (see the kernel above).
+  const int n_tiles = p.counts[1];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((threadIdx.x >> 6) & 3);
+  const bool producer = threadIdx.x < 256;
+  const int half = lane >> 5, col = lane & 31;
+  const int ac = p.attend_current;
+  const int wph = p.wgs_per_head;
+  int head, w;
+  if ((p.num_heads & 7) == 0) {
+    const int hpx = p.num_heads >> 3, r0 = blockIdx.x >> 3;
+    head = (blockIdx.x & 7) * hpx + r0 % hpx;
+    w = r0 / hpx;
+  } else {
+    head = blockIdx.x % p.num_heads;
+    w = blockIdx.x / p.num_heads;
+  }
+  int* next_slot_lds = reinterpret_cast<int*>(lds_raw + (size_t)Lds::kElems * sizeof(T));
+  auto first_row_block = [&](const Tile& tl) {               // first 32-row step that sees the tile's first key
+    const int first_row = tl.origin + 1 - ac;
+    return first_row < tl.seq_len ? (first_row / kRows) * kRows : tl.seq_len;
+  };
+  Tile next_tile = p.k_tiles[w < n_tiles ? w : 0];
+
+  if (producer) {
+    const int g = wave;                                      // this wave's 32-key sub-tile of the tile
+    // K and V of the sub-tile as MFMA A operands, stationary in registers.  The next tile's are requested into the
+    // same registers as soon as the last MFMAs of this tile have been issued.
+    vec8 kf[kSteps], vf[kSteps];
+    auto load_kv = [&](const Tile& tl) {
+      const T* kb = (const T*)p.k.ptr + tl.seq_id * p.k.sb + head * p.k.sh + (int64_t)tl.seq_start * p.k.st;
+      const T* vb = (const T*)p.v.ptr + tl.seq_id * p.v.sb + head * p.v.sh + (int64_t)tl.seq_start * p.v.st;
+      const int key = tl.origin + 32 * g + mfma_row_to_key32(col);
+      const RowSource<T> ks = make_row_source<T, true>(kb, p.k.st, tl.seq_len, DH), vs = make_row_source<T, true>(vb, p.v.st, tl.seq_len, DH);
+#pragma unroll
+      for (int kk = 0; kk < kSteps; kk++) {       // keys beyond the sequence are outside the buffer and read as zero
+        kf[kk] = as_vec8<T>(__builtin_amdgcn_raw_buffer_load_b128(ks.rsrc, key * ks.stride_bytes + (16 * kk + 8 * half) * (int)sizeof(T), 0, 0));
+        vf[kk] = as_vec8<T>(__builtin_amdgcn_raw_buffer_load_b128(vs.rsrc, key * vs.stride_bytes + (16 * kk + 8 * half) * (int)sizeof(T), 0, 0));
+      }
+    };
+    if (w < n_tiles) load_kv(next_tile);
+    for (int slot = w; slot < n_tiles;) {
+      const Tile tile = next_tile;
+      if (threadIdx.x == 0) *next_slot_lds = wph + atomicAdd(p.head_queue + head, 1);
+      const int L = tile.seq_len, j0 = tile.origin;
+      const int64_t tok0 = tile.seq_start;
+      const int jt = j0 / kDkv4Keys;
+      const int first_row = j0 + 1 - ac;                     // first row that sees key j0
+      const int n_qt = (L + kBlockQ - 1) / kBlockQ;
+      const int row_begin = first_row < L ? (first_row / kRows) * kRows : L;
+      const int n_steps = (L - row_begin + kRows - 1) / kRows;
+      const int jb = j0 + 32 * g;                            // first key of this wave's sub-tile
+      const int64_t slot0 = (int64_t)head * p.carry_head_stride + tile.carry_base +
+                            carry_offset(4 * jt + g, n_qt) - (int64_t)kBlockQ * jt;      // + row
+      const float* carry = p.carry + slot0;
+      const float* prefix = p.prefix + slot0;
+      const float* drem_eff = p.drem_eff + tile.seq_id * p.stat_sb + head * p.stat_sh + tok0;
+      // Per-row scalars (drem, product above the sub-tile, C below it), fetched two steps ahead: a step is shorter
+      // than a global load.
+      float n_drem = 0.f, n_prod = 1.f, n_prefix = 0.f, nn_drem = 0.f, nn_prod = 1.f, nn_prefix = 0.f;
+      auto fetch_row_scalars = [&](int row0, float& drem_r, float& prod_r, float& prefix_r) {
+        const int r = row0 + col;
+        drem_r = r < L ? drem_eff[r] : 0.f;
+        prod_r = carry[r];
+        prefix_r = prefix[r];
+      };
+      if (n_steps > 0) fetch_row_scalars(row_begin, n_drem, n_prod, n_prefix);
+      if (n_steps > 1) fetch_row_scalars(row_begin + kRows, nn_drem, nn_prod, nn_prefix);
+      lds_barrier();                                         // rows of steps 0 and 1 are in LDS; the queue slot too
+      slot = *next_slot_lds;                                 // the tile after this one
+      const bool have_next = slot < n_tiles;
+      if (have_next) next_tile = p.k_tiles[slot];
+
+      // S^T and dP^T of the rows in stage `st` against this wave's sub-tile.
+      auto scores = [&](int st, f32x16& s, f32x16& dp) {
+        const T* q_lds = lds + Lds::kQ + st * 2 * Lds::kQdoTile;
+        const T* do_lds = q_lds + Lds::kQdoTile;
+#pragma unroll
+        for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
+        {
+          vec8 bq[kSteps];
+#pragma unroll
+          for (int kk = 0; kk < kSteps; kk++) bq[kk] = lds_row8<T>(q_lds, kRowStride, col, 16 * kk + 8 * half);
+#pragma unroll
+          for (int kk = 0; kk < kSteps; kk++) s = Elem<T>::mfma(kf[kk], bq[kk], s);
+        }
+        {
+          vec8 bdo[kSteps];
+#pragma unroll
+          for (int kk = 0; kk < kSteps; kk++) bdo[kk] = lds_row8<T>(do_lds, kRowStride, col, 16 * kk + 8 * half);
+#pragma unroll
+          for (int kk = 0; kk < kSteps; kk++) dp = Elem<T>::mfma(vf[kk], bdo[kk], dp);
+        }
+      };
+      // The math of one step on (s_cur, dp_cur) with the MFMAs of the next step (rows in stage `st`, results in
+      // s_next / dp_next) dealt among it, so that the matrix pipe runs under the vector ALU instead of stalling the
+      // wave.  The block is one scheduling region whose issue order is spelled out at the end: the Q operands are
+      // requested first and the first elements' math covers their latency, then one MFMA per kGap vector-ALU
+      // instructions, with the dO operands requested a few MFMAs in.
+      auto fused = [&](auto diag_tag, int st, const f32x16& s_cur, const f32x16& dp_cur, f32x16& s_next, f32x16& dp_next,
+                       int lim, float drem, float prod_in, float prefix_in, uint32_t (&pk)[8], uint32_t (&dzk)[8]) {
+        constexpr bool kDiag = decltype(diag_tag)::value;
+        constexpr int kLead = 24;                              // vector-ALU instructions ahead of the first MFMA
+        constexpr int kGap = (kDiag ? 270 : 230) / (2 * kSteps);
+        constexpr int kAlu = 0x402;                            // scheduling-group mask: vector ALU incl. transcendentals
+        const T* q_lds = lds + Lds::kQ + st * 2 * Lds::kQdoTile;
+        const T* do_lds = q_lds + Lds::kQdoTile;
+        __builtin_amdgcn_sched_barrier(0);
+        vec8 bq[kSteps], bdo[kSteps];
+#pragma unroll
+        for (int kk = 0; kk < kSteps; kk++) bq[kk] = lds_row8<T>(q_lds, kRowStride, col, 16 * kk + 8 * half);
+#pragma unroll
+        for (int kk = 0; kk < kSteps; kk++) bdo[kk] = lds_row8<T>(do_lds, kRowStride, col, 16 * kk + 8 * half);
+#pragma unroll
+        for (int r = 0; r < 16; r++) { s_next[r] = 0.f; dp_next[r] = 0.f; }
+#pragma unroll
+        for (int kk = 0; kk < kSteps; kk++) s_next = Elem<T>::mfma(kf[kk], bq[kk], s_next);
+#pragma unroll
+        for (int kk = 0; kk < kSteps; kk++) dp_next = Elem<T>::mfma(vf[kk], bdo[kk], dp_next);
+        f32x16 sc[1], dpc[1];
+        sc[0] = s_cur; dpc[0] = dp_cur;
+        float prod_lower, prefix_upper, prefix_next;
+        bwd_tile_math_impl<T, 1, kDiag>(sc, dpc, p.scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prod_lower,
+                                        prefix_upper, prefix_next);
+        __builtin_amdgcn_sched_group_barrier(0x100, kSteps, 0);
+        __builtin_amdgcn_sched_group_barrier(kAlu, kLead, 0);
+#pragma unroll
+        for (int i = 0; i < 2 * kSteps; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kAlu, kGap, 0);
+          if (i == kSteps / 2 - 1) __builtin_amdgcn_sched_group_barrier(0x100, kSteps, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      // One step: P^T / dZ^T of step t to LDS, S^T / dP^T of step t+1 into the other pair of accumulators.
+      auto step = [&](int t, f32x16& s_cur, f32x16& dp_cur, f32x16& s_next, f32x16& dp_next) {
+        if (t >= n_steps) return;
+        const int q0 = row_begin + t * kRows;
+        const float drem = n_drem, prod_in = n_prod, prefix_in = n_prefix;
+        n_drem = nn_drem; n_prod = nn_prod; n_prefix = nn_prefix;
+        if (t + 2 < n_steps) fetch_row_scalars(q0 + 2 * kRows, nn_drem, nn_prod, nn_prefix);
+        const int w_last = q0 + kRows - 1;
+        const int qi = q0 + col;
+        const bool row_ok = qi < L;
+        const int st_next = (t + 1) & 3;
+        uint32_t pk[8], dzk[8];
+        const int lim = row_ok ? qi + ac - jb - 16 * half : 0;
+        if (jb > w_last - 1 + ac || jb >= L) {               // nothing of this sub-tile is visible to these rows
+          scores(st_next, s_next, dp_next);
+#pragma unroll
+          for (int i = 0; i < 8; i++) { pk[i] = 0; dzk[i] = 0; }
+        } else if ((jb + 31) > (q0 - 1 + ac) || w_last >= L) {
+          fused(std::true_type{}, st_next, s_cur, dp_cur, s_next, dp_next, lim, drem, prod_in, prefix_in, pk, dzk);
+        } else {
+          fused(std::false_type{}, st_next, s_cur, dp_cur, s_next, dp_next, lim, drem, prod_in, prefix_in, pk, dzk);
+        }
+        // [query][key] tiles: this lane's 16 consecutive keys start at column 32*g + 16*half of row `col`.
+        T* p_lds = lds + Lds::kP + (t & 1) * 2 * Lds::kPTile;
+        u32x4* pp = reinterpret_cast<u32x4*>(p_lds + col * kPStride + 32 * g + 16 * half);
+        u32x4* dd = reinterpret_cast<u32x4*>(p_lds + Lds::kPTile + col * kPStride + 32 * g + 16 * half);
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+          pp[c] = u32x4{pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
+          dd[c] = u32x4{dzk[4 * c], dzk[4 * c + 1], dzk[4 * c + 2], dzk[4 * c + 3]};
+        }
+        if (t == n_steps - 1 && have_next) load_kv(next_tile);   // kf / vf have fed their last MFMAs of this tile
+      };
+      f32x16 s_a, dp_a, s_b, dp_b;
+      if (n_steps > 0) scores(0, s_a, dp_a);
+      else if (have_next) load_kv(next_tile);
+      for (int t = 0; t <= n_steps; t += 2) {
+        step(t, s_a, dp_a, s_b, dp_b);
+        lds_barrier();
+        if (t + 1 <= n_steps) {
+          step(t + 1, s_b, dp_b, s_a, dp_a);
+          lds_barrier();
+        }
+      }
+    }  // tile walk (producers)
+  } else {
+    constexpr int kCT = DH / 64;                             // 32-column blocks per consumer wave
+    const int mp = wave >> 1, cp = wave & 1;                 // keys 64*mp .. +63, columns 32*kCT*cp .. +32*kCT-1
+    f32x16 dkacc[2][kCT], dvacc[2][kCT];
+    // Two sets of staging registers, used alternately: a step's rows are requested two steps before they are
+    // written to LDS (a step is shorter than a global load).
+    TileCopy<T, DH, kRows, true> cq[2], cdo[2];
+    auto stage_first = [&](const Tile& tl) {                 // rows of steps 0 and 1 of a tile
+      const T* qb = (const T*)p.q.ptr + tl.seq_id * p.q.sb + head * p.q.sh + (int64_t)tl.seq_start * p.q.st;
+      const T* dob = (const T*)p.d_o.ptr + tl.seq_id * p.d_o.sb + head * p.d_o.sh + (int64_t)tl.seq_start * p.d_o.st;
+      const RowSource<T> qs = make_row_source<T, true>(qb, p.q.st, tl.seq_len, DH), ds = make_row_source<T, true>(dob, p.d_o.st, tl.seq_len, DH);
+      const int rb = first_row_block(tl);
+#pragma unroll
+      for (int i = 0; i < 2; i++)                            // rows beyond the sequence read as zero
+        if (rb + i * kRows < tl.seq_len) {
+          cq[i].load(qs, rb + i * kRows);
+          cdo[i].load(ds, rb + i * kRows);
+        }
+    };
+    if (w < n_tiles) stage_first(next_tile);
+    // The results of a tile are stored during the first step of the NEXT tile, when the consumers have nothing to
+    // contract yet (and after the last tile): acc[m][n][r] is key origin + 64*mp + 32*m + 8*(r/4) + 4*half + r%4,
+    // column 32*(kCT*cp + n) + col.
+    bool pending = false;
+    Tile done_tile = next_tile;
+    auto store_results = [&](const Tile& tl) {
+      const int tl_len = tl.seq_len, tl_j0 = tl.origin + 64 * mp;
+      const int64_t tl_tok0 = tl.seq_start;
+      T* dkb = (T*)p.dk.ptr + tl.seq_id * p.dk.sb + head * p.dk.sh + tl_tok0 * p.dk.st;
+      T* dvb = (T*)p.dv.ptr + tl.seq_id * p.dv.sb + head * p.dv.sh + tl_tok0 * p.dv.st;
+      if (p.add_rem) {
+        // the remainder term o += rem * v contributes rem_j * d_o_j to dv_j
+        const T* dob = (const T*)p.d_o.ptr + tl.seq_id * p.d_o.sb + head * p.d_o.sh + tl_tok0 * p.d_o.st;
+#pragma unroll
+        for (int m = 0; m < 2; m++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int key = tl_j0 + 32 * m + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (key < tl_len) {
+              const float rem = fast_exp2(p.row_stat[tl.seq_id * p.stat_sb + head * p.stat_sh + tl_tok0 + key]);
+#pragma unroll
+              for (int n = 0; n < kCT; n++)
+                dvacc[m][n][r] += rem * (float)dob[(int64_t)key * p.d_o.st + 32 * (kCT * cp + n) + col];
+            }
+          }
+      }
+      const RowSink<T> dk_sink = make_row_sink<T>(dkb, p.dk.st, tl_len, DH), dv_sink = make_row_sink<T>(dvb, p.dv.st, tl_len, DH);
+      T* scratch = lds + Lds::kScratch + wave * (32 * lds_stride<32>());
+#pragma unroll
+      for (int m = 0; m < 2; m++)
+#pragma unroll
+        for (int n = 0; n < kCT; n++) {
+          store_acc_tile_wide<T>(dk_sink, dkacc[m][n], p.logit_scale, tl_j0 + 32 * m, 32 * (kCT * cp + n), half, col, lane, scratch);
+          store_acc_tile_wide<T>(dv_sink, dvacc[m][n], 1.f, tl_j0 + 32 * m, 32 * (kCT * cp + n), half, col, lane, scratch);
+        }
+    };
+    for (int slot = w; slot < n_tiles;) {
+      const Tile tile = next_tile;
+      const int L = tile.seq_len, j0 = tile.origin;
+      const int64_t tok0 = tile.seq_start;
+      const int first_row = j0 + 1 - ac;
+      const int row_begin = first_row < L ? (first_row / kRows) * kRows : L;
+      const int n_steps = (L - row_begin + kRows - 1) / kRows;
+      const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
+      const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
+      const RowSource<T> qsrc = make_row_source<T, true>(qb, p.q.st, L, DH), dosrc = make_row_source<T, true>(dob, p.d_o.st, L, DH);
+      // Rows of step r into stage r%4 from register set r%2, then the rows of step r+2 requested into that set.
+      auto stage_rows = [&](int r) {
+        T* q_lds = lds + Lds::kQ + (r & 3) * 2 * Lds::kQdoTile;
+        const int rn = row_begin + (r + 2) * kRows;
+        if (r & 1) {
+          cq[1].store(q_lds); cdo[1].store(q_lds + Lds::kQdoTile);
+          if (rn < L) { cq[1].load(qsrc, rn); cdo[1].load(dosrc, rn); }
+        } else {
+          cq[0].store(q_lds); cdo[0].store(q_lds + Lds::kQdoTile);
+          if (rn < L) { cq[0].load(qsrc, rn); cdo[0].load(dosrc, rn); }
+        }
+      };
+      stage_rows(0);
+      stage_rows(1);
+      lds_barrier();
+      slot = *next_slot_lds;                                 // the tile after this one
+      const bool have_next = slot < n_tiles;
+      if (have_next) next_tile = p.k_tiles[slot];
+      // Step 0: nothing to contract yet, so the previous tile's results leave now.
+      if (pending) store_results(done_tile);
+      stage_rows(2);
+#pragma unroll
+      for (int m = 0; m < 2; m++)
+#pragma unroll
+        for (int n = 0; n < kCT; n++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) { dkacc[m][n][r] = 0.f; dvacc[m][n][r] = 0.f; }
+      lds_barrier();
+      for (int t = 1; t <= n_steps; ++t) {
+        stage_rows(t + 2);
+        const int u = t - 1;
+        const T* q_lds = lds + Lds::kQ + (u & 3) * 2 * Lds::kQdoTile;
+        const T* do_lds = q_lds + Lds::kQdoTile;
+        const T* p_lds = lds + Lds::kP + (u & 1) * 2 * Lds::kPTile;
+        const T* dz_lds = p_lds + Lds::kPTile;
+        // dV[key][d] += sum_i P[i][key] dO[i][d];  dK[key][d] += sum_i dZ[i][key] Q[i][d]   (i over the 32 rows)
+#pragma unroll
+        for (int c = 0; c < kRows / 16; c++) {
+          const int row0 = 16 * c + 8 * half;
+          vec8 ap[2], az[2], bd[kCT], bq[kCT];
+#pragma unroll
+          for (int m = 0; m < 2; m++) {
+            ap[m] = lds_col8<T>(p_lds, kPStride, row0, 64 * mp + 32 * m, lane);
+            az[m] = lds_col8<T>(dz_lds, kPStride, row0, 64 * mp + 32 * m, lane);
+          }
+#pragma unroll
+          for (int n = 0; n < kCT; n++) {
+            bd[n] = lds_col8<T>(do_lds, kRowStride, row0, 32 * (kCT * cp + n), lane);
+            bq[n] = lds_col8<T>(q_lds, kRowStride, row0, 32 * (kCT * cp + n), lane);
+          }
+#pragma unroll
+          for (int m = 0; m < 2; m++)
+#pragma unroll
+            for (int n = 0; n < kCT; n++) {
+              dvacc[m][n] = Elem<T>::mfma(ap[m], bd[n], dvacc[m][n]);
+              dkacc[m][n] = Elem<T>::mfma(az[m], bq[n], dkacc[m][n]);
+            }
+        }
+        lds_barrier();
+      }
+      // The next tile's first rows are requested before this tile's results are stored.
+      if (have_next) stage_first(next_tile);
+      pending = true;
+      done_tile = tile;
+    }  // tile walk (consumers)
+    if (pending) store_results(done_tile);
+  }
+}
+
+template <typename T, int DH>
+static hipError_t launch_dkv4(const BwdParams& p_in, int max_tiles, hipStream_t stream) {
+  const size_t lds_bytes = (size_t)Dkv4Lds<DH>::kElems * sizeof(T) + 256;      // + the published queue slot
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv4_kernel<T, DH>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+  if (e != hipSuccess) return e;
+  int dev = 0, cus = 0;
+  if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+  if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+  BwdParams p = p_in;
+  p.wgs_per_head = cus / p.num_heads > 0 ? cus / p.num_heads : 1;
+  if (p.wgs_per_head > max_tiles) p.wgs_per_head = max_tiles;
+  const dim3 grid((unsigned)(p.wgs_per_head * p.num_heads)), block(kDkv4Threads);
+  hipLaunchKernelGGL((bwd_dkv4_kernel<T, DH>), grid, block, lds_bytes, stream, p);
+  return hipGetLastError();
+}
+
 template <typename T, int DH, bool kFast>
 static hipError_t launch_one(const BwdParams& p, int max_tiles, hipStream_t stream) {
   const size_t lds_bytes = (size_t)DkvLds<DH>::kElems * sizeof(T);
@@ -530,9 +907,20 @@ static hipError_t launch_one(const BwdParams& p, int max_tiles, hipStream_t stre
 
 template <typename T>
 static hipError_t launch_t(const BwdParams& p, int max_tiles, hipStream_t stream) {
+#ifndef SBA_DKV3_ONLY
+  if (p.vec_ok && p.head_dim == 128) return launch_dkv4<T, 128>(p, max_tiles, stream);
+#endif
   if (p.vec_ok && p.head_dim == 128) return launch_dkv3<T, 128>(p, max_tiles, stream);
   if (p.vec_ok && p.head_dim == 64) return launch_dkv3<T, 64>(p, max_tiles, stream);
   return p.head_dim <= 64 ? launch_one<T, 64, false>(p, max_tiles, stream) : launch_one<T, 128, false>(p, max_tiles, stream);
+}
+
+// Keys per key tile of the kernel launch_bwd_dkv will pick for these parameters.
+int dkv_key_tile(const BwdParams& p) {
+#ifndef SBA_DKV3_ONLY
+  if (p.vec_ok && p.head_dim == 128) return kDkv4Keys;
+#endif
+  return kBlockK;
 }
 
 hipError_t launch_bwd_dkv(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream) {

@@ -31,11 +31,12 @@ struct SchedParams {
   int32_t want_key_tiles;  // backward: also build the key-tile list
   int32_t want_carry_base; // also lay out the per-sequence carry offsets
   Tile* q_tiles;           // query tiles (kBlockQ rows), heaviest first
-  Tile* k_tiles;           // key tiles (kBlockK keys), heaviest first
+  Tile* k_tiles;           // key tiles (key_tile keys), heaviest first
   int32_t* counts;         // [0] = number of query tiles, [1] = number of key tiles
   int64_t* carry_base;     // per sequence: first carry slot of the sequence (per head)
   int32_t* head_queue;     // backward: per-head cursor into the key-tile list, reset to 0 here
   int32_t num_heads;
+  int32_t key_tile;        // keys per key tile (a multiple of 32; what the dK/dV kernel that will run sweeps)
 };
 
 struct FwdParams {

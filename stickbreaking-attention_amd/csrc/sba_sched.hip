@@ -27,17 +27,6 @@ __device__ __forceinline__ void seq_bounds(const SchedParams& p, int s, int* sta
   *start = (int)beg;
   *len = (int)(end > beg ? end - beg : 0);
 }
-// Number of key tiles a query tile sweeps.
-__device__ __forceinline__ int q_tile_work(int q0, int len, int ac) {
-  const int last_key = min(q0 + kBlockQ, len) - 2 + ac;
-  return last_key < 0 ? 0 : last_key / kBlockK + 1;
-}
-// Number of query tiles a key tile is swept by.
-__device__ __forceinline__ int k_tile_work(int j0, int len, int ac) {
-  const int first_row = j0 + 1 - ac;
-  if (first_row >= len) return 0;
-  return (len + kBlockQ - 1) / kBlockQ - first_row / kBlockQ;
-}
 
 // Exclusive prefix sum over bins taken from the heaviest bin downwards; bins[] becomes the start offsets.
 __device__ void descending_offsets(int* bins, int* scratch) {
@@ -75,7 +64,7 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
   for (int s = threadIdx.x; s < p.num_seqs; s += kSchedThreads) {
     int start, len;
     seq_bounds(p, s, &start, &len);
-    const int nq = (len + kBlockQ - 1) / kBlockQ, nk = (len + kBlockK - 1) / kBlockK;
+    const int nq = (len + kBlockQ - 1) / kBlockQ, nk = (len + p.key_tile - 1) / p.key_tile;
     const int cls = min(nq, kBins - 1);
     if (nq) atomicAdd(&qbins[cls], nq);
     if (nk && p.want_key_tiles) atomicAdd(&kbins[cls], nk);
@@ -115,7 +104,7 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
   for (int s = wave; s < p.num_seqs; s += nwaves) {
     int start, len;
     seq_bounds(p, s, &start, &len);
-    const int nq = (len + kBlockQ - 1) / kBlockQ, nk = (len + kBlockK - 1) / kBlockK;
+    const int nq = (len + kBlockQ - 1) / kBlockQ, nk = (len + p.key_tile - 1) / p.key_tile;
     const int cls = min(nq, kBins - 1);
     int qbase = 0, kbase = 0;
     if (lane == 0) {
@@ -131,7 +120,7 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
     }
     if (p.want_key_tiles) {
       for (int t = lane; t < nk; t += 64) {      // heaviest key tile (the first one) first
-        Tile d; d.seq_start = start; d.seq_len = len; d.origin = t * kBlockK; d.seq_id = s; d.carry_base = cbase;
+        Tile d; d.seq_start = start; d.seq_len = len; d.origin = t * p.key_tile; d.seq_id = s; d.carry_base = cbase;
         p.k_tiles[kbase + t] = d;
       }
     }
