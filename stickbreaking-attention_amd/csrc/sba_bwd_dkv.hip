@@ -188,7 +188,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// head_dim 128 fast path: producer / consumer waves.
+// Fast path, producer / consumer waves (runs head_dim 64; head_dim 128 runs the software-pipelined kernel below).
 //
 // One workgroup = 8 waves = one 64-key tile, swept by query tiles of 64 rows.  Waves 0-3 are PRODUCERS: wave
 // (rg, g) takes rows 32*rg .. +31 against the 32-key sub-tile g (one MFMA row tile, 16 keys per lane, that
@@ -907,20 +907,15 @@ static hipError_t launch_one(const BwdParams& p, int max_tiles, hipStream_t stre
 
 template <typename T>
 static hipError_t launch_t(const BwdParams& p, int max_tiles, hipStream_t stream) {
-#ifndef SBA_DKV3_ONLY
+  // head_dim 64 measures slightly faster on the 64-key kernel (its steps are already short).
   if (p.vec_ok && p.head_dim == 128) return launch_dkv4<T, 128>(p, max_tiles, stream);
-#endif
-  if (p.vec_ok && p.head_dim == 128) return launch_dkv3<T, 128>(p, max_tiles, stream);
   if (p.vec_ok && p.head_dim == 64) return launch_dkv3<T, 64>(p, max_tiles, stream);
   return p.head_dim <= 64 ? launch_one<T, 64, false>(p, max_tiles, stream) : launch_one<T, 128, false>(p, max_tiles, stream);
 }
 
 // Keys per key tile of the kernel launch_bwd_dkv will pick for these parameters.
 int dkv_key_tile(const BwdParams& p) {
-#ifndef SBA_DKV3_ONLY
-  if (p.vec_ok && p.head_dim == 128) return kDkv4Keys;
-#endif
-  return kBlockK;
+  return (p.vec_ok && p.head_dim == 128) ? kDkv4Keys : kBlockK;
 }
 
 hipError_t launch_bwd_dkv(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream) {
