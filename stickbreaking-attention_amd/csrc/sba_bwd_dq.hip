@@ -17,6 +17,8 @@
 #include "sba_device.hpp"
 #include "sba_params.hpp"
 
+#include <type_traits>
+
 namespace sba {
 
 template <typename T, int DH, bool kFast, int KT>
@@ -123,27 +125,54 @@ __global__ __launch_bounds__(kThreads, KT == 32 ? 2 : 1) void bwd_dq_kernel(BwdP
     const bool diagonal = (j0 + KT - 1) > (w_first - 1 + ac) || w_last >= L;
 
     f32x16 s[NT], dp[NT];
-#pragma unroll
-    for (int mt = 0; mt < NT; mt++) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) { s[mt][r] = 0.f; dp[mt][r] = 0.f; }
-      const int krow = NT == 2 ? mfma_row_to_key(mt, col) : mfma_row_to_key32(col);
-#pragma unroll
-      for (int kk = 0; kk < kSteps; kk++) {
-        vec8 a = lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half);
-        s[mt] = Elem<T>::mfma(a, qf[kk], s[mt]);
-      }
-#pragma unroll
-      for (int kk = 0; kk < kSteps; kk++) {
-        vec8 a = lds_row8<T>(v_lds, kRowStride, krow, 16 * kk + 8 * half);
-        dp[mt] = Elem<T>::mfma(a, dof[kk], dp[mt]);
-      }
-    }
     const int lim = row_ok ? qi + ac - j0 - (KT / 2) * half : 0;
     uint32_t pk[8 * NT], dzk[8 * NT];
     float prod_lower, prefix_upper;
-    bwd_tile_math<T, NT>(s, dp, p.scale_log2, diagonal, lim, half, drem, prod_in, prefix, pk, dzk, prod_lower,
-                         prefix_upper, prefix);
+    if (NT == 1 && kFast) {
+      // 32-key steps: S^T first; the dP^T MFMAs are dealt among the element-wise math (its first phase only needs
+      // S), one MFMA per kGap vector-ALU instructions, so that the matrix pipe runs under the vector ALU.
+      const int krow = mfma_row_to_key32(col);
+#pragma unroll
+      for (int r = 0; r < 16; r++) { s[0][r] = 0.f; dp[0][r] = 0.f; }
+#pragma unroll
+      for (int kk = 0; kk < kSteps; kk++) s[0] = Elem<T>::mfma(lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half), qf[kk], s[0]);
+      auto math = [&](auto diag_tag) {
+        constexpr bool kDiag = decltype(diag_tag)::value;
+        constexpr int kGap = 96 / kSteps;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < kSteps; kk++) dp[0] = Elem<T>::mfma(lds_row8<T>(v_lds, kRowStride, krow, 16 * kk + 8 * half), dof[kk], dp[0]);
+        bwd_tile_math_impl<T, NT, kDiag>(s, dp, p.scale_log2, lim, half, drem, prod_in, prefix, pk, dzk, prod_lower, prefix_upper, prefix);
+        __builtin_amdgcn_sched_group_barrier(0x100, kSteps, 0);
+        __builtin_amdgcn_sched_group_barrier(0x402, 8, 0);
+#pragma unroll
+        for (int kk = 0; kk < kSteps; kk++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x402, kGap, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      if (diagonal) math(std::true_type{}); else math(std::false_type{});
+    } else {
+#pragma unroll
+      for (int mt = 0; mt < NT; mt++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) { s[mt][r] = 0.f; dp[mt][r] = 0.f; }
+        const int krow = NT == 2 ? mfma_row_to_key(mt, col) : mfma_row_to_key32(col);
+#pragma unroll
+        for (int kk = 0; kk < kSteps; kk++) {
+          vec8 a = lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half);
+          s[mt] = Elem<T>::mfma(a, qf[kk], s[mt]);
+        }
+#pragma unroll
+        for (int kk = 0; kk < kSteps; kk++) {
+          vec8 a = lds_row8<T>(v_lds, kRowStride, krow, 16 * kk + 8 * half);
+          dp[mt] = Elem<T>::mfma(a, dof[kk], dp[mt]);
+        }
+      }
+      bwd_tile_math<T, NT>(s, dp, p.scale_log2, diagonal, lim, half, drem, prod_in, prefix, pk, dzk, prod_lower,
+                           prefix_upper, prefix);
+    }
     if (NT == 2 && half == 0) prefix_out[slot_hi] = prefix_upper;
 
     // dQ += dZ K: A = dZ from registers, B = K gathered down the keys.
