@@ -665,7 +665,7 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
                        int lim, float drem, float prod_in, float prefix_in, uint32_t (&pk)[8], uint32_t (&dzk)[8]) {
         constexpr bool kDiag = decltype(diag_tag)::value;
         constexpr int kLead = 24;                              // vector-ALU instructions ahead of the first MFMA
-        constexpr int kGap = (kDiag ? 270 : 230) / (2 * kSteps);
+        constexpr int kGap = (kDiag ? 270 : 240) / (2 * kSteps);
         constexpr int kAlu = 0x402;                            // scheduling-group mask: vector ALU incl. transcendentals
         const T* q_lds = lds + Lds::kQ + st * 2 * Lds::kQdoTile;
         const T* do_lds = q_lds + Lds::kQdoTile;
@@ -698,7 +698,10 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
       };
       // One step: P^T / dZ^T of step t to LDS, S^T / dP^T of step t+1 into the other pair of accumulators.
       auto step = [&](int t, f32x16& s_cur, f32x16& dp_cur, f32x16& s_next, f32x16& dp_next) {
-        if (t >= n_steps) return;
+        if (t >= n_steps) {                                  // the consumers' last step: only the barrier of the step before
+          if (t > 0) lds_barrier();
+          return;
+        }
         const int q0 = row_begin + t * kRows;
         const float drem = n_drem, prod_in = n_prod, prefix_in = n_prefix;
         n_drem = nn_drem; n_prod = nn_prod; n_prefix = nn_prefix;
@@ -709,6 +712,10 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
         const int st_next = (t + 1) & 3;
         uint32_t pk[8], dzk[8];
         const int lim = row_ok ? qi + ac - jb - 16 * half : 0;
+        // The barrier that ends the previous step is met here, behind this step's bookkeeping, which covers the
+        // latency of the previous step's P / dZ writes.
+        __builtin_amdgcn_sched_barrier(0);
+        if (t > 0) lds_barrier();
         if (jb > w_last - 1 + ac || jb >= L) {               // nothing of this sub-tile is visible to these rows
           scores(st_next, s_next, dp_next);
 #pragma unroll
@@ -734,12 +741,9 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
       else if (have_next) load_kv(next_tile);
       for (int t = 0; t <= n_steps; t += 2) {
         step(t, s_a, dp_a, s_b, dp_b);
-        lds_barrier();
-        if (t + 1 <= n_steps) {
-          step(t + 1, s_b, dp_b, s_a, dp_a);
-          lds_barrier();
-        }
+        if (t + 1 <= n_steps) step(t + 1, s_b, dp_b, s_a, dp_a);
       }
+      lds_barrier();                                         // the barrier of the last step
     }  // tile walk (producers)
   } else {
     constexpr int kCT = DH / 64;                             // 32-column blocks per consumer wave
