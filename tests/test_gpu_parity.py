@@ -82,6 +82,7 @@ SMALL = [
     ("d127-unaligned", 3, 127, [70, 1, 130]),
     ("300-singletons", 2, 8, [1] * 300),
     ("d24-tile-edges", 5, 24, [33, 64, 63, 65, 127, 128, 129]),
+    ("d128-tile-edges", 3, 128, [31, 32, 33, 127, 255, 256, 257, 383, 385, 2, 97]),
 ]
 
 
