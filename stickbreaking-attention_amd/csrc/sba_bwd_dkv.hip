@@ -665,6 +665,9 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
                        int lim, float drem, float prod_in, float prefix_in, uint32_t (&pk)[8], uint32_t (&dzk)[8]) {
         constexpr bool kDiag = decltype(diag_tag)::value;
         constexpr int kLead = 24;                              // vector-ALU instructions ahead of the first MFMA
+        // Vector-ALU instructions per MFMA.  The group solver is greedy: with a budget a little below the block's
+        // instruction count it puts the last MFMAs back to back and the rest of the math behind them, so the values
+        // were checked in the generated code (both element types, both copies of the unrolled step).
         constexpr int kGap = (kDiag ? 270 : 240) / (2 * kSteps);
         constexpr int kAlu = 0x402;                            // scheduling-group mask: vector ALU incl. transcendentals
         const T* q_lds = lds + Lds::kQ + st * 2 * Lds::kQdoTile;
