@@ -142,7 +142,7 @@ __global__ __launch_bounds__(kThreads, KT == 32 ? 2 : 1) void bwd_dq_kernel(BwdP
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int kk = 0; kk < kSteps; kk++) dp[0] = Elem<T>::mfma(lds_row8<T>(v_lds, kRowStride, krow, 16 * kk + 8 * half), dof[kk], dp[0]);
-        bwd_tile_math_impl<T, NT, kDiag>(s, dp, p.scale_log2, lim, half, drem, prod_in, prefix, pk, dzk, prod_lower, prefix_upper, prefix);
+        bwd_tile_math_impl<T, NT, kDiag, false>(s, dp, p.scale_log2, lim, half, drem, prod_in, prefix, pk, dzk, prod_lower, prefix_upper, prefix);
         __builtin_amdgcn_sched_group_barrier(0x100, kSteps, 0);
         __builtin_amdgcn_sched_group_barrier(0x402, 8, 0);
 #pragma unroll
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(kThreads, KT == 32 ? 2 : 1) void bwd_dq_kernel(BwdP
           dp[mt] = Elem<T>::mfma(a, dof[kk], dp[mt]);
         }
       }
-      bwd_tile_math<T, NT>(s, dp, p.scale_log2, diagonal, lim, half, drem, prod_in, prefix, pk, dzk, prod_lower,
+      bwd_tile_math<T, NT, false>(s, dp, p.scale_log2, diagonal, lim, half, drem, prod_in, prefix, pk, dzk, prod_lower,
                            prefix_upper, prefix);
     }
     if (NT == 2 && half == 0) prefix_out[slot_hi] = prefix_upper;

@@ -218,7 +218,7 @@ __device__ __forceinline__ u32x4 load_row8(const T* row, int d0, int d_valid, bo
 // Produces P (pk) and dZ = g - sigma * C (dzk), C_ij = sum_{j' <= j} g_ij', packed to 16 bit two keys per
 // word, and the prefix sum for the next tile up.  (The reference evaluates the same quantities tile by tile at
 // stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:438-447.)
-template <typename T, int NT, bool kDiagonal>
+template <typename T, int NT, bool kDiagonal, bool kNeedP = true>
 __device__ __forceinline__ void bwd_tile_math_impl(const f32x16 (&s)[NT], const f32x16 (&dp)[NT], float scale_log2, int lim,
                                                    int half, float drem, float prod_in, float prefix_in,
                                                    uint32_t (&pk)[8 * NT], uint32_t (&dzk)[8 * NT], float& prod_lower,
@@ -244,13 +244,20 @@ __device__ __forceinline__ void bwd_tile_math_impl(const f32x16 (&s)[NT], const 
   // share of the lower half-wave's total is added afterwards (fixup).
   float acc = prefix_in;
   float dz[N];
+  const float neg_drem_seed = -drem * seed;
 #pragma unroll
   for (int R = 0; R < N; R++) {
-    const float a = beta[R] * (pe[R] * seed);
-    const float g = a * (dp[R >> 4][R & 15] - drem);
+    float g;
+    if (kNeedP) {
+      const float a = beta[R] * (pe[R] * seed);
+      g = a * (dp[R >> 4][R & 15] - drem);
+      pe[R] = a;
+    } else {
+      // A is not wanted for itself: the seed goes into (dP - drem) with one fma instead of a multiply of its own
+      g = (beta[R] * pe[R]) * fmaf(dp[R >> 4][R & 15], seed, neg_drem_seed);
+    }
     acc += g;
     dz[R] = g - beta[R] * acc;
-    pe[R] = a;
   }
   const float tot = acc - prefix_in;
   const float oth_g = other_half(tot, half);
@@ -259,23 +266,23 @@ __device__ __forceinline__ void bwd_tile_math_impl(const f32x16 (&s)[NT], const 
   prefix_out = acc + oth_g;
 #pragma unroll
   for (int R = 0; R < N; R += 2) {
-    pk[R >> 1] = pack2<T>(pe[R], pe[R + 1]);
+    pk[R >> 1] = kNeedP ? pack2<T>(pe[R], pe[R + 1]) : 0u;
     dzk[R >> 1] = pack2<T>(dz[R] - beta[R] * fixup, dz[R + 1] - beta[R + 1] * fixup);
   }
 }
 
 // prod_lower / prefix_upper: the same two carries at the boundary between the two half-waves' keys (the middle of
 // the tile), for consumers that work on half the keys at a time.
-template <typename T, int NT>
+template <typename T, int NT, bool kNeedP = true>
 __device__ __forceinline__ void bwd_tile_math(const f32x16 (&s)[NT], const f32x16 (&dp)[NT], float scale_log2, bool diagonal,
                                               int lim, int half, float drem, float prod_in, float prefix_in,
                                               uint32_t (&pk)[8 * NT], uint32_t (&dzk)[8 * NT], float& prod_lower,
                                               float& prefix_upper, float& prefix_out) {
   if (diagonal)
-    bwd_tile_math_impl<T, NT, true>(s, dp, scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prod_lower,
+    bwd_tile_math_impl<T, NT, true, kNeedP>(s, dp, scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prod_lower,
                                     prefix_upper, prefix_out);
   else
-    bwd_tile_math_impl<T, NT, false>(s, dp, scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prod_lower,
+    bwd_tile_math_impl<T, NT, false, kNeedP>(s, dp, scale_log2, lim, half, drem, prod_in, prefix_in, pk, dzk, prod_lower,
                                      prefix_upper, prefix_out);
 }
 
