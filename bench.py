@@ -32,7 +32,7 @@ MFMA_BF16_PEAK = 2.5e15          # MI355X dense bf16 MFMA peak, FLOP/s
 # `--pmc WRITE_SIZE` runs of `bench.py --traffic-probe`, each scaled by what the same counter read for the probe's
 # 1 GiB device-to-device copy.  Hardware counters cannot be read from inside this script, so the figures are carried
 # here; they are reported only for the workload they were measured on.
-MEASURED_TRAFFIC_BYTES = {"c3": {"fwd_kernel": 2.051e9, "bwd_dq_kernel": 1.980e9, "bwd_dkv_kernel": 2.619e9}}
+MEASURED_TRAFFIC_BYTES = {"c3": {"fwd_kernel": 2.059e9, "bwd_dq_kernel": 1.950e9, "bwd_dkv_kernel": 2.616e9}}
 
 
 # ----------------------------------------------------------------------------------------------
