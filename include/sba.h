@@ -18,8 +18,16 @@
  *   - Packed (varlen) mode: cu_seqlens != NULL, tensors are (H, T, D), batch stride ignored.
  *     Fixed-length mode: cu_seqlens == NULL, tensors are (B, H, L, D) with num_seqs = B and
  *     total_tokens = L.
- *   - Re-entrant and stream-ordered; no global mutable state.  Calls that share a workspace must
- *     be ordered on one stream.
+ *   - Re-entrant and stream-ordered.  The only process-wide state is a per-device cache of device
+ *     attributes (compute-unit count, the kernels' LDS limits), filled on first use.  Calls that
+ *     share a workspace must be ordered on one stream.
+ *   - cu_seqlens is read on the device, so a bad one cannot be reported by the return value.  The
+ *     scheduler checks every entry (non-decreasing, within [0, total_tokens], a leading entry equal
+ *     to 0) and that the carry buffer is large enough for the actual lengths; on failure it schedules
+ *     nothing, all outputs of the call are zero-filled, and the int32 at SBA_STATUS_OFFSET of the
+ *     workspace holds SBA_SCHED_BAD_CU_SEQLENS or SBA_SCHED_CARRY_TOO_SMALL (0 otherwise) once the
+ *     stream has run.  Rows of the packed token axis at or beyond the last cu_seqlens entry belong to
+ *     no sequence; their outputs and gradients are zero-filled.
  */
 #ifndef SBA_H
 #define SBA_H
@@ -31,7 +39,13 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 2
+#define SBA_VERSION 3
+
+/* Scheduler status word: int32 at this byte offset of the workspace, valid after the stream has run. */
+#define SBA_STATUS_OFFSET 8
+#define SBA_SCHED_OK 0
+#define SBA_SCHED_BAD_CU_SEQLENS 1
+#define SBA_SCHED_CARRY_TOO_SMALL 2
 
 typedef enum SbaDtype { SBA_BF16 = 0, SBA_F32 = 1, SBA_F16 = 2 } SbaDtype;
 
@@ -40,10 +54,11 @@ typedef enum SbaStatus {
   SBA_ERR_NULL = -1,        /* a required pointer is NULL */
   SBA_ERR_DTYPE = -2,       /* dtype not supported by this build */
   SBA_ERR_HEAD_DIM = -3,    /* head_dim outside 1..128 */
-  SBA_ERR_STRIDE = -4,      /* a row (token) or head stride is not a multiple of the vector width, or negative */
-  SBA_ERR_ALIGN = -5,       /* a tensor base pointer is not 16-byte aligned */
-  SBA_ERR_SHAPE = -6,       /* non-positive sizes */
-  SBA_ERR_WORKSPACE = -7,   /* workspace missing or smaller than sba_workspace_bytes reports */
+  SBA_ERR_STRIDE = -4,      /* a negative stride (any non-negative head/token/batch stride is accepted; strides and
+                               base pointers that are multiples of 16 bytes select the fast kernels) */
+  SBA_ERR_ALIGN = -5,       /* a tensor base pointer is not aligned to its element size */
+  SBA_ERR_SHAPE = -6,       /* non-positive sizes, total_tokens > 2^30, or a reserved field that is not 0 */
+  SBA_ERR_WORKSPACE = -7,   /* workspace missing, not 256-byte aligned, or smaller than sba_workspace_bytes reports */
   SBA_ERR_LAUNCH = -8       /* the HIP runtime rejected a launch (hipGetLastError) */
 } SbaStatus;
 
@@ -102,7 +117,24 @@ typedef struct SbaArgs {
                                   gradient that reaches rem directly, needs row_stat (as the forward wrote it) as an
                                   input, and returns dv including rem * d_o. */
   int32_t reserved0;           /* must be 0 */
+  int64_t carry_slots;         /* fp32 slots of `carry` (and of the backward's prefix plane) per head.  0: sized from
+                                  the bound total_tokens * max_seqlen / 64 (packed mode), which is several times the
+                                  need of a ragged batch; a caller that knows the lengths on the host passes
+                                  SbaPlan.carry_slots from sba_plan_host for the exact size.  Must be the same in the
+                                  forward, the backward and sba_workspace_bytes. */
 } SbaArgs;
+
+/* What the device scheduler will derive from cu_seqlens, computed on the host from a host copy. */
+typedef struct SbaPlan {
+  int32_t status;              /* SBA_SCHED_OK or SBA_SCHED_BAD_CU_SEQLENS, as the device scheduler would decide */
+  int32_t longest;             /* longest sequence */
+  int64_t covered_tokens;      /* tokens that belong to a sequence (the last cu_seqlens entry) */
+  int64_t query_tiles;         /* 128-row query tiles over all sequences */
+  int64_t key_tiles;           /* 64-key tiles over all sequences */
+  int64_t carry_slots;         /* exact fp32 slots per head of the carry buffer: sum over sequences of
+                                  256 M (M + 1), M = ceil(length / 128) */
+  int64_t pairs;               /* visible (query, key) pairs per head */
+} SbaPlan;
 
 /* ABI version of this header (SBA_VERSION) the library was built against. */
 int sba_version(void);
@@ -119,6 +151,17 @@ const char* sba_strerror(int status);
 int sba_workspace_bytes(const SbaArgs* args, size_t* fwd_bytes, size_t* bwd_bytes, size_t* carry_bytes);
 
 /*
+ * Host mirror of the device scheduler's reading of cu_seqlens (same code): validates a HOST copy of
+ * cu_seqlens (element width and leading zero as args->cu_is_int64 / cu_has_leading_zero say; num_seqs,
+ * total_tokens, attend_current from args) and reports the exact sizes.  Touches no device.  For callers
+ * that have the lengths on the host anyway and want exact buffer sizes, and for validating cu_seqlens
+ * before a launch.  In fixed-length mode (cu_seqlens_host == NULL) the plan is that of num_seqs
+ * sequences of total_tokens.  The reference has no counterpart (its grid is padded to max_seqlens:
+ * sb_varlen_fwd.py:475-479, and cu_seqlens is not validated: sb_varlen_fwd.py:283-288).
+ */
+int sba_plan_host(const SbaArgs* args, const void* cu_seqlens_host, SbaPlan* plan);
+
+/*
  * Forward: fills o, rem, row_stat (and carry when given).
  * Replaces `_compileable_forward` (stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:453-521,
  * custom op "varlen_fwd") and `_compileable_fwd` (stickbreaking_attention/sb_attn/sb_fwd.py:175-251,
@@ -128,8 +171,10 @@ int sba_workspace_bytes(const SbaArgs* args, size_t* fwd_bytes, size_t* bwd_byte
 int sba_fwd(const SbaArgs* args);
 
 /*
- * Backward: fills dq, dk, dv from q, k, v, carry, d_o, d_rem (and row_stat when add_remainder is set).  Every element of dq, dk, dv is written
- * exactly once (no zero-fill needed, no atomics, no locks).
+ * Backward: fills dq, dk, dv from q, k, v, carry, d_o, d_rem (and row_stat when add_remainder is set).
+ * 16-bit dtypes: every element of dq, dk, dv is written exactly once (no zero-fill needed, no atomics,
+ * no locks; bit-reproducible).  SBA_F32: dk and dv are zero-filled by the call and summed with fp32
+ * atomics, so their last bits depend on the execution order.
  * Replaces `_compileable_backward` (stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:541-640,
  * custom op "varlen_bwd") and (stickbreaking_attention/sb_attn/sb_bwd.py:207-296, custom op
  * "attn_bwd"), and the `locked_add` accumulation (sb_varlen_bwd.py:11-53).

@@ -21,6 +21,13 @@ What it restates (citations are into the reference repository):
   form dz_ij = g_ij - sigmoid(z_ij) * sum_{j'<=j} g_ij', g_ij = A_ij (do_i.v_j - drem_i), which is
   what stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:438-452 evaluates tile by tile.
 
+* ``rounding_floor``           -- the streaming form evaluated in float64 with exactly two kinds of rounding
+  put back: the weights P and the logit gradient dZ are rounded to the 16-bit input type before they are
+  contracted (the reference rounds at the same points: sb_varlen_fwd.py:193 ``p.to(v.dtype)``,
+  sb_varlen_bwd.py:449-450 ``dqk.to(k.dtype)``), and the five results are rounded to the 16-bit output type.
+  It is the error no implementation with 16-bit matrix operands and 16-bit outputs can avoid; the GPU tests
+  compare the kernels' error with it on the same inputs.
+
 Parity status: every function here is pinned by tests/test_oracle_pins.py against checks that do
 not retype its formula -- an O(L^3) scalar-loop evaluation of the product form
 A_ij = s_ij * prod_{j<k<i}(1 - s_ik) in float64, the q = 0 closed form (A_ij = 2^-(i-j),
@@ -200,6 +207,55 @@ def dense_backward_autograd(q, k, v, cu_seqlens, do, drem, scale=None, zero_star
     o, rem = varlen_dense(q, k, v, cu_seqlens, scale, zero_start, attend_current)
     torch.autograd.backward([o, rem], [do, drem])
     return o.detach(), rem.detach(), q.grad, k.grad, v.grad
+
+
+def rounding_floor(q, k, v, do, drem, scale=None, attend_current=False, low=torch.bfloat16, with_exact=False):
+    """(o, rem, dq, dk, dv) of one (L, D) problem as an implementation would return them that computes everything
+    exactly (float64 here) except that P and dZ are rounded to ``low`` before their contractions and the outputs are
+    rounded to ``low``.  Inputs are the ``low``-rounded values both sides consume.  ``with_exact`` also returns the
+    unrounded float64 results from the same intermediates (what ``stream_forward`` / ``stream_backward`` give)."""
+    q, k, v, do, drem = (t.double() for t in (q, k, v, do, drem))
+    if scale is None:
+        scale = 1.0 / math.sqrt(q.shape[-1])
+    rnd = lambda t: t.to(low).double()
+    o, rem, att, beta = stream_forward(q, k, v, scale, attend_current, want_att=True)
+    g = torch.matmul(do, v.transpose(-1, -2))
+    g -= drem[..., None]
+    g *= att
+    dz = g.cumsum(-1)
+    dz *= beta
+    del beta
+    torch.sub(g, dz, out=dz)
+    del g
+    dz.masked_fill_(~_visible(q.shape[-2], attend_current, q.device), 0)
+    exact = (o, rem, scale * torch.matmul(dz, k), scale * torch.matmul(dz.transpose(-1, -2), q),
+             torch.matmul(att.transpose(-1, -2), do)) if with_exact else None
+    p16, dz16 = rnd(att), rnd(dz)
+    del att, dz
+    floor = (rnd(torch.matmul(p16, v)), rnd(rem), rnd(scale * torch.matmul(dz16, k)),
+             rnd(scale * torch.matmul(dz16.transpose(-1, -2), q)), rnd(torch.matmul(p16.transpose(-1, -2), do)))
+    return (floor, exact) if with_exact else floor
+
+
+def varlen_rounding_floor(q, k, v, cu_seqlens, do, drem, scale=None, zero_start=False, attend_current=False,
+                          heads: Optional[Sequence[int]] = None, low=torch.bfloat16):
+    """``rounding_floor`` over a packed (H, T, D) batch, one (head, sequence) slice at a time.  Returns
+    ``(floor, exact)``: two (o, rem, dq, dk, dv) tuples in float64 (heads outside ``heads`` are zeros)."""
+    ends = _normalise_cu(cu_seqlens, zero_start)
+    H, T, D = q.shape
+    heads = range(H) if heads is None else heads
+    make = lambda: [torch.zeros(H, T, D, dtype=torch.float64), torch.zeros(H, T, dtype=torch.float64)] + \
+                   [torch.zeros(H, T, D, dtype=torch.float64) for _ in range(3)]
+    floor, exact = make(), make()
+    for h in heads:
+        start = 0
+        for end in ends:
+            sl = slice(start, end)
+            f, e = rounding_floor(q[h, sl], k[h, sl], v[h, sl], do[h, sl], drem[h, sl], scale, attend_current, low, with_exact=True)
+            for dst, src in zip(floor + exact, f + e):
+                dst[h, sl] = src
+            start = end
+    return tuple(floor), tuple(exact)
 
 
 def with_remainder(outputs, v, do=None):

@@ -33,6 +33,7 @@ int plan(const SbaArgs* a, Layout* out) {
   if (a->head_dim < 1 || a->head_dim > 128) return SBA_ERR_HEAD_DIM;
   if (a->dtype != SBA_BF16 && a->dtype != SBA_F16 && a->dtype != SBA_F32) return SBA_ERR_DTYPE;
   if (a->total_tokens > (int64_t)1 << 30) return SBA_ERR_SHAPE;
+  if (a->reserved0 != 0 || a->carry_slots < 0) return SBA_ERR_SHAPE;
   Layout L{};
   const int64_t T = a->total_tokens, B = a->num_seqs;
   const bool fixed = a->cu_seqlens == nullptr;
@@ -47,6 +48,8 @@ int plan(const SbaArgs* a, Layout* out) {
     // sum_s 256 M_s (M_s + 1) with M_s <= L_s/128 + 1 and sum_s L_s^2 <= T * max_len
     L.carry_slots_per_head = cdiv(T * max_len, 64) + 6 * T + 512 * B;
   }
+  // A caller that knows the lengths passes the exact count (sba_plan_host); the scheduler checks it on the device.
+  if (a->carry_slots > 0) L.carry_slots_per_head = a->carry_slots;
   size_t off = 0;
   L.off_counts = off;      off = align_up(off + 256, 256);
   L.off_q_tiles = off;     off = align_up(off + (size_t)L.max_q_tiles * sizeof(sba::Tile), 256);
@@ -91,6 +94,8 @@ int run_sched(const SbaArgs* a, const Layout& L, bool want_key_tiles, bool want_
   sp.cu_has_leading_zero = a->cu_has_leading_zero;
   sp.num_seqs = a->num_seqs;
   sp.fixed_len = (int32_t)a->total_tokens;
+  sp.total_tokens = a->total_tokens;
+  sp.carry_capacity = L.carry_slots_per_head;
   sp.attend_current = a->attend_current ? 1 : 0;
   sp.want_key_tiles = want_key_tiles ? 1 : 0;
   sp.want_carry_base = want_carry_base ? 1 : 0;
@@ -136,6 +141,31 @@ int sba_workspace_bytes(const SbaArgs* args, size_t* fwd_bytes, size_t* bwd_byte
   return SBA_OK;
 }
 
+int sba_plan_host(const SbaArgs* a, const void* cu_host, SbaPlan* out) {
+  if (!a || !out) return SBA_ERR_NULL;
+  if (a->num_seqs <= 0 || a->total_tokens <= 0 || a->total_tokens > (int64_t)1 << 30) return SBA_ERR_SHAPE;
+  SbaPlan pl{};
+  const int ac = a->attend_current ? 1 : 0;
+  for (int s = 0; s < a->num_seqs; s++) {
+    int32_t start = 0, len = (int32_t)a->total_tokens;
+    if (cu_host && !sba::seq_span(cu_host, a->cu_is_int64, a->cu_has_leading_zero, s, a->total_tokens, &start, &len))
+      pl.status = SBA_SCHED_BAD_CU_SEQLENS;
+    const int64_t n = len, m = cdiv(n, kBlockQ);
+    pl.query_tiles += m;
+    pl.key_tiles += cdiv(n, kBlockK);
+    pl.carry_slots += sba::carry_slots(m);
+    pl.pairs += n * (n - 1) / 2 + (ac ? n : 0);
+    if (len > pl.longest) pl.longest = len;
+    pl.covered_tokens = cu_host ? (int64_t)start + len : a->total_tokens;
+  }
+  if (pl.status != SBA_SCHED_OK) {      // the device scheduler voids the whole schedule
+    pl.query_tiles = pl.key_tiles = pl.carry_slots = pl.pairs = pl.covered_tokens = 0;
+    pl.longest = 0;
+  }
+  *out = pl;
+  return SBA_OK;
+}
+
 int sba_fwd(const SbaArgs* a) {
   if (!a) return SBA_ERR_NULL;
   Layout L;
@@ -170,9 +200,11 @@ int sba_fwd(const SbaArgs* a) {
   p.scale_log2 = (float)((double)a->logit_scale * kLog2e);
   p.attend_current = a->attend_current ? 1 : 0;
   p.add_rem = a->add_remainder ? 1 : 0;
+  p.max_tiles = (int32_t)L.max_q_tiles;
+  p.total_tokens = a->total_tokens;
   const int64_t max_rows = (a->max_seqlen > 0 && a->max_seqlen < a->total_tokens) ? a->max_seqlen : a->total_tokens;
   bool v16 = (a->head_dim % (16 / (int)es)) == 0;
-  for (const SbaTensor* t : {&a->q, &a->k, &a->v}) v16 = v16 && vec16(*t, es, fixed, max_rows);
+  for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->o}) v16 = v16 && vec16(*t, es, fixed, max_rows);
   p.vec_ok = v16 ? 1 : 0;
   hipEvent_t* ev = (hipEvent_t*)a->trace_events;
   if (ev && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;
@@ -226,6 +258,8 @@ int sba_bwd(const SbaArgs* a) {
   p.stat_sh = a->total_tokens;
   p.drem_eff = (float*)(ws + L.off_drem);
   p.head_queue = (int32_t*)(ws + L.off_queue);
+  p.max_tiles = (int32_t)L.max_q_tiles;
+  p.total_tokens = a->total_tokens;
   const int64_t max_rows = (a->max_seqlen > 0 && a->max_seqlen < a->total_tokens) ? a->max_seqlen : a->total_tokens;
   bool v16 = (a->head_dim % (16 / (int)es)) == 0;
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})

@@ -14,9 +14,34 @@
 #include "sba_device.hpp"
 #include "sba_params.hpp"
 
+#include <atomic>
 #include <type_traits>
 
 namespace sba {
+
+// Launch facts that do not change while the process lives, looked up once per device instead of on every call:
+// the compute-unit count, and which kernels have had their dynamic-LDS limit raised on which device.
+static hipError_t device_cus(int* dev_out, int* cus_out) {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  int cus = (dev >= 0 && dev < 64) ? cached[dev].load(std::memory_order_relaxed) : 0;
+  if (cus == 0) {
+    if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+    if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
+  }
+  *dev_out = dev; *cus_out = cus;
+  return hipSuccess;
+}
+template <typename Kernel>
+static hipError_t raise_lds_limit(Kernel kernel, std::atomic<uint64_t>& done, int dev, size_t lds_bytes) {
+  const uint64_t bit = (dev >= 0 && dev < 64) ? (uint64_t)1 << dev : 0;
+  if (bit && (done.load(std::memory_order_acquire) & bit)) return hipSuccess;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+  if (e == hipSuccess && bit) done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
 
 template <int DH> struct DkvLds {
   static constexpr int kRowStride = lds_stride<DH>();
@@ -109,8 +134,8 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
     const int qi = w_first + col;
     const bool row_ok = qi < L;
     uint32_t pk[16], dzk[16];
-    if (j0 > w_last - 1 + ac) {
-      // no row of this wave sees the tile: contributes zeros
+    if (j0 > min(w_last, L - 1) - 1 + ac) {
+      // no row of this wave that belongs to the sequence sees the tile: contributes zeros
 #pragma unroll
       for (int i = 0; i < 16; i++) { pk[i] = 0; dzk[i] = 0; }
     } else {
@@ -333,7 +358,10 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
         const int qi = w_first + col;
         const bool row_ok = qi < L;
         uint32_t pk[8], dzk[8];
-        if (jb > w_last - 1 + ac || jb >= L) {
+        // Skipped unless a row of the SEQUENCE sees the sub-tile: the forward and the dQ kernel record the per-row
+        // scalars only for sub-tiles that hold a key visible to the last row of their query tile, so a sub-tile that
+        // merely lies below rows beyond the sequence's end has no recorded values to start from.
+        if (jb > min(w_last, L - 1) - 1 + ac) {
 #pragma unroll
           for (int i = 0; i < 8; i++) { pk[i] = 0; dzk[i] = 0; }
         } else {
@@ -501,13 +529,12 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
 template <typename T, int DH>
 static hipError_t launch_dkv3(const BwdParams& p_in, int max_tiles, hipStream_t stream) {
   const size_t lds_bytes = (size_t)Dkv3Lds<DH>::kElems * sizeof(T) + 256;      // + the published queue slot
-  // The tile set exceeds the default 64 KB dynamic-LDS cap; the attribute is per device and cheap to set.
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv3_kernel<T, DH>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-  if (e != hipSuccess) return e;
+  // The tile set exceeds the default 64 KB dynamic-LDS cap: the limit is raised once per device.
+  static std::atomic<uint64_t> lds_done{0};
   int dev = 0, cus = 0;
-  if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
-  if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+  hipError_t e = device_cus(&dev, &cus);
+  if (e != hipSuccess) return e;
+  if ((e = raise_lds_limit(&bwd_dkv3_kernel<T, DH>, lds_done, dev, lds_bytes)) != hipSuccess) return e;
   BwdParams p = p_in;
   // One workgroup per CU: the same number of workgroups for every head, and with a head count that is a multiple of
   // 8 the workgroups of a head share an XCD (workgroup ids are dealt round-robin to the 8 XCDs).
@@ -719,7 +746,8 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
         // latency of the previous step's P / dZ writes.
         __builtin_amdgcn_sched_barrier(0);
         if (t > 0) lds_barrier();
-        if (jb > w_last - 1 + ac || jb >= L) {               // nothing of this sub-tile is visible to these rows
+        if (jb > min(w_last, L - 1) - 1 + ac) {              // no row of the sequence in this step sees the sub-tile (and
+                                                             // no per-row scalars were recorded for it)
           scores(st_next, s_next, dp_next);
 #pragma unroll
           for (int i = 0; i < 8; i++) { pk[i] = 0; dzk[i] = 0; }
@@ -886,12 +914,11 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
 template <typename T, int DH>
 static hipError_t launch_dkv4(const BwdParams& p_in, int max_tiles, hipStream_t stream) {
   const size_t lds_bytes = (size_t)Dkv4Lds<DH>::kElems * sizeof(T) + 256;      // + the published queue slot
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv4_kernel<T, DH>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-  if (e != hipSuccess) return e;
+  static std::atomic<uint64_t> lds_done{0};
   int dev = 0, cus = 0;
-  if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
-  if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+  hipError_t e = device_cus(&dev, &cus);
+  if (e != hipSuccess) return e;
+  if ((e = raise_lds_limit(&bwd_dkv4_kernel<T, DH>, lds_done, dev, lds_bytes)) != hipSuccess) return e;
   BwdParams p = p_in;
   p.wgs_per_head = cus / p.num_heads > 0 ? cus / p.num_heads : 1;
   if (p.wgs_per_head > max_tiles) p.wgs_per_head = max_tiles;
@@ -903,10 +930,11 @@ static hipError_t launch_dkv4(const BwdParams& p_in, int max_tiles, hipStream_t 
 template <typename T, int DH, bool kFast>
 static hipError_t launch_one(const BwdParams& p, int max_tiles, hipStream_t stream) {
   const size_t lds_bytes = (size_t)DkvLds<DH>::kElems * sizeof(T);
-  // The tile set exceeds the default 64 KB dynamic-LDS cap; the attribute is per device and cheap to set.
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_dkv_kernel<T, DH, kFast>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+  static std::atomic<uint64_t> lds_done{0};
+  int dev = 0, cus = 0;
+  hipError_t e = device_cus(&dev, &cus);
   if (e != hipSuccess) return e;
+  if ((e = raise_lds_limit(&bwd_dkv_kernel<T, DH, kFast>, lds_done, dev, lds_bytes)) != hipSuccess) return e;
   const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kThreads);
   hipLaunchKernelGGL((bwd_dkv_kernel<T, DH, kFast>), grid, block, lds_bytes, stream, p);
   return hipGetLastError();

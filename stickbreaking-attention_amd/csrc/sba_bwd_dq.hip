@@ -33,7 +33,15 @@ __global__ __launch_bounds__(kThreads, KT == 32 ? 2 : 1) void bwd_dq_kernel(BwdP
 
   int head, slot;
   xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
-  if (slot >= p.counts[0]) return;
+  if (slot >= p.counts[kCountQ]) {
+    int64_t r0, r1;
+    if (uncovered_rows(p.counts, slot, p.total_tokens, 0, kBlockQ, &r0, &r1)) {      // rows of no sequence: zero gradients
+      zero_rows<T>(p.dq, head, r0, r1, p.head_dim);
+      zero_rows<T>(p.dk, head, r0, r1, p.head_dim);
+      zero_rows<T>(p.dv, head, r0, r1, p.head_dim);
+    }
+    return;
+  }
   const Tile tile = p.q_tiles[slot];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, col = lane & 31;
   const int L = tile.seq_len, q0 = tile.origin, ac = p.attend_current, D = p.head_dim;

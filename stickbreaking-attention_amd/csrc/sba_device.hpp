@@ -340,6 +340,24 @@ __device__ __forceinline__ void store_acc_tile_wide(const RowSink<T>& sink, cons
   }
 }
 
+// Rows of the packed token axis that belong to no sequence (total_tokens beyond the last cu_seqlens entry, or every
+// row when the scheduler voided the schedule) are zero-filled by the workgroups that find no tile: idle slot
+// `slot - counts[kCountQ]` of a head clears `rows` rows of that head starting at counts[kCountCovered].  The launch
+// provides ceil(total_tokens / 128) + num_seqs slots per head, which leaves at least ceil(uncovered / 128) idle.
+// (The reference allocates zero-filled gradients and rem: sb_varlen_bwd.py:506-508, sb_varlen_fwd.py:418.)
+__device__ __forceinline__ bool uncovered_rows(const int32_t* counts, int slot, int64_t total_tokens, int sub, int rows,
+                                               int64_t* r0, int64_t* r1) {
+  *r0 = (int64_t)counts[kCountCovered] + (int64_t)kBlockQ * (slot - counts[kCountQ]) + (int64_t)sub * rows;
+  *r1 = *r0 + rows < total_tokens ? *r0 + rows : total_tokens;
+  return *r0 < *r1;
+}
+template <typename T>
+__device__ __forceinline__ void zero_rows(const TensorRef& t, int head, int64_t r0, int64_t r1, int d) {
+  T* b = (T*)t.ptr + head * t.sh;
+  const int64_t n = (r1 - r0) * d;
+  for (int64_t idx = threadIdx.x; idx < n; idx += blockDim.x) b[(r0 + idx / d) * t.st + idx % d] = (T)0;
+}
+
 // Map the linear workgroup id to (head, tile slot) so that the workgroups of one head land on one XCD
 // (workgroups are dealt round-robin to the 8 XCDs, each with a private L2): K/V of a head are then
 // re-read from that XCD's L2 rather than from HBM.

@@ -56,7 +56,17 @@ __global__ __launch_bounds__(kThreads) void fwd_f32_kernel(FwdParams p) {
   __shared__ float q_lds[kWaves][kMaxD];
   int head, slot;
   xcd_head_tile(blockIdx.x / kF32Split, p.num_heads, &head, &slot);
-  if (slot >= p.counts[0]) return;
+  if (slot >= p.counts[kCountQ]) {
+    int64_t r0, r1;
+    if (uncovered_rows(p.counts, slot, p.total_tokens, blockIdx.x % kF32Split, kF32Rows, &r0, &r1)) {
+      zero_rows<float>(p.o, head, r0, r1, p.head_dim);      // rows of no sequence: o = rem = 0
+      for (int64_t r = r0 + threadIdx.x; r < r1; r += kThreads) {
+        ((float*)p.rem.ptr)[head * p.rem.sh + r * p.rem.st] = 0.f;
+        p.row_stat[head * p.stat_sh + r] = 0.f;
+      }
+    }
+    return;
+  }
   const Tile tile = p.tiles[slot];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int row_base = tile.origin + (blockIdx.x % kF32Split) * kF32Rows + wave * kF32RowsPerWave;
@@ -135,7 +145,7 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_kernel(BwdParams p) {
   BwdF32Lds& lds = *reinterpret_cast<BwdF32Lds*>(lds_raw);
   int head, slot;
   xcd_head_tile(blockIdx.x / kF32Split, p.num_heads, &head, &slot);
-  if (slot >= p.counts[0]) return;
+  if (slot >= p.counts[kCountQ]) return;
   const Tile tile = p.q_tiles[slot];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wg_row0 = tile.origin + (blockIdx.x % kF32Split) * kF32Rows;      // first row of this workgroup
@@ -246,6 +256,8 @@ hipError_t launch_fwd_f32(const FwdParams& p, int max_tiles, hipStream_t stream)
 hipError_t launch_bwd_f32(const BwdParams& p, int batches, int64_t tokens, int max_q_tiles, hipStream_t stream) {
   hipLaunchKernelGGL(fill_zero_rows_kernel, dim3(1024), dim3(256), 0, stream, p.dk, batches, p.num_heads, tokens, p.head_dim);
   hipLaunchKernelGGL(fill_zero_rows_kernel, dim3(1024), dim3(256), 0, stream, p.dv, batches, p.num_heads, tokens, p.head_dim);
+  // dq is stored, not accumulated, but only for rows that belong to a sequence: the fill covers the others.
+  hipLaunchKernelGGL(fill_zero_rows_kernel, dim3(1024), dim3(256), 0, stream, p.dq, batches, p.num_heads, tokens, p.head_dim);
   if (hipGetLastError() != hipSuccess) return hipErrorLaunchFailure;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_f32_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(BwdF32Lds));

@@ -30,7 +30,17 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
 
   int head, slot;
   xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
-  if (slot >= p.counts[0]) return;
+  if (slot >= p.counts[kCountQ]) {
+    int64_t r0, r1;
+    if (uncovered_rows(p.counts, slot, p.total_tokens, 0, kBlockQ, &r0, &r1)) {      // rows of no sequence: o = rem = 0
+      zero_rows<T>(p.o, head, r0, r1, p.head_dim);
+      for (int64_t r = r0 + threadIdx.x; r < r1; r += kThreads) {
+        ((T*)p.rem.ptr)[head * p.rem.sh + r * p.rem.st] = (T)0;
+        p.row_stat[head * p.stat_sh + r] = 0.f;
+      }
+    }
+    return;
+  }
   const Tile tile = p.tiles[slot];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, col = lane & 31;
   const int L = tile.seq_len, q0 = tile.origin, ac = p.attend_current, D = p.head_dim;
@@ -66,6 +76,10 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
     ck.load(ksrc, (n_kt - 1) * KT);
     cv.load(vsrc, (n_kt - 1) * KT);
   }
+  // The recorded products are read per 64-key tile by the backward kernels that sweep 64 keys at a time, whichever
+  // forward variant ran: a 32-key sweep that ends on the lower half of such a tile also records the (empty) product
+  // above the upper half.
+  if (NT == 1 && carry && half == 0 && (n_kt & 1)) carry[carry_offset(n_kt, n_qt) + (qi - kBlockQ * (n_kt >> 2))] = 1.f;
   for (int jt = n_kt - 1; jt >= 0; --jt) {
     const int j0 = jt * KT;
     __syncthreads();

@@ -22,17 +22,25 @@ struct Tile {
   int64_t carry_base;  // first carry slot of the sequence within a head's plane (0 when no carries are laid out)
 };
 
+// Slots of the scheduler's `counts` array.
+enum : int { kCountQ = 0, kCountK = 1, kCountStatus = 2, kCountCovered = 3 };
+// Values of counts[kCountStatus].
+enum : int { kSchedOk = 0, kSchedBadCu = 1, kSchedCarryOverflow = 2 };
+
 struct SchedParams {
   const void* cu;          // NULL: fixed-length mode
   int32_t cu_is_int64, cu_has_leading_zero;
   int32_t num_seqs;
   int32_t fixed_len;       // L in fixed-length mode
+  int64_t total_tokens;    // T: rows of the packed token axis (L in fixed-length mode)
+  int64_t carry_capacity;  // carry slots reserved per head
   int32_t attend_current;
   int32_t want_key_tiles;  // backward: also build the key-tile list
   int32_t want_carry_base; // also lay out the per-sequence carry offsets
   Tile* q_tiles;           // query tiles (kBlockQ rows), heaviest first
   Tile* k_tiles;           // key tiles (key_tile keys), heaviest first
-  int32_t* counts;         // [0] = number of query tiles, [1] = number of key tiles
+  int32_t* counts;         // [kCountQ] query tiles, [kCountK] key tiles, [kCountStatus], [kCountCovered] = tokens
+                           // covered by sequences (rows at or beyond it belong to no sequence and are zero-filled)
   int64_t* carry_base;     // per sequence: first carry slot of the sequence (per head)
   int32_t* head_queue;     // backward: per-head cursor into the key-tile list, reset to 0 here
   int32_t num_heads;
@@ -54,6 +62,8 @@ struct FwdParams {
   int32_t attend_current;
   int32_t vec_ok;              // all row strides / base pointers allow 16-byte accesses and head_dim % 8 == 0
   int32_t add_rem;             // write o + rem * v
+  int32_t max_tiles;           // query-tile slots the launch provides per head (>= counts[kCountQ])
+  int64_t total_tokens;        // packed mode: rows of the token axis; rows no sequence covers are zero-filled
 };
 
 struct BwdParams {
@@ -79,7 +89,24 @@ struct BwdParams {
   int32_t* head_queue;         // per head: next key tile not yet taken (beyond the first wgs_per_head), zero at launch
   float* drem_eff;             // workspace, indexed like row_stat: the gradient of rem per row in fp32 (d_rem, plus
                                // d_o . v when add_rem), written by the dQ kernel and read by the dK/dV kernel
+  int32_t max_tiles;           // query-tile slots the dQ launch provides per head
+  int64_t total_tokens;        // packed mode: rows of the token axis; rows no sequence covers are zero-filled
 };
+
+// One sequence's token range from cu_seqlens (cumulative sequence ends, optionally preceded by a 0).  Returns false
+// when the entry is unusable: ends must be non-decreasing, within [0, total_tokens], and a leading entry must be 0.
+// The reference reads the same two entries without any check (sb_varlen_fwd.py:283-288); here a bad entry voids the
+// whole schedule instead of sending tiles outside the tensors.  Shared by the device scheduler and its host mirror.
+__host__ __device__ inline bool seq_span(const void* cu, int is_int64, int leading_zero, int s, int64_t total_tokens,
+                                         int32_t* start, int32_t* len) {
+  const int idx = s + (leading_zero ? 1 : 0);
+  const int64_t end = is_int64 ? ((const int64_t*)cu)[idx] : (int64_t)((const int32_t*)cu)[idx];
+  const int64_t beg = idx == 0 ? 0 : (is_int64 ? ((const int64_t*)cu)[idx - 1] : (int64_t)((const int32_t*)cu)[idx - 1]);
+  const bool ok = beg >= 0 && beg <= end && end <= total_tokens && !(leading_zero && s == 0 && beg != 0);
+  *start = ok ? (int32_t)beg : 0;
+  *len = ok ? (int32_t)(end - beg) : 0;
+  return ok;
+}
 
 // Carry slots.  Carries are kept per (row, 32-key sub-tile): sub-tile U covers keys 32U .. 32U+31 of the
 // sequence and is needed by the rows of query tiles U/4, U/4 + 1, ..., M-1 (M = query tiles of 128 rows the

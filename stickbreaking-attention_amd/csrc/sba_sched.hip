@@ -16,16 +16,10 @@ namespace sba {
 constexpr int kBins = 4096;          // sequence length classes (query tiles per sequence, saturating)
 constexpr int kSchedThreads = 1024;
 
-__device__ __forceinline__ int64_t read_cu(const SchedParams& p, int idx) {
-  return p.cu_is_int64 ? ((const int64_t*)p.cu)[idx] : (int64_t)((const int32_t*)p.cu)[idx];
-}
-__device__ __forceinline__ void seq_bounds(const SchedParams& p, int s, int* start, int* len) {
-  if (p.cu == nullptr) { *start = 0; *len = p.fixed_len; return; }
-  const int off = p.cu_has_leading_zero ? 1 : 0;
-  const int64_t end = read_cu(p, s + off);
-  const int64_t beg = (s + off == 0) ? 0 : read_cu(p, s + off - 1);
-  *start = (int)beg;
-  *len = (int)(end > beg ? end - beg : 0);
+// Returns false for an unusable cu_seqlens entry (see seq_span); the span is then empty.
+__device__ __forceinline__ bool seq_bounds(const SchedParams& p, int s, int* start, int* len) {
+  if (p.cu == nullptr) { *start = 0; *len = p.fixed_len; return true; }
+  return seq_span(p.cu, p.cu_is_int64, p.cu_has_leading_zero, s, p.total_tokens, start, len);
 }
 
 // Exclusive prefix sum over bins taken from the heaviest bin downwards; bins[] becomes the start offsets.
@@ -55,21 +49,30 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
   __shared__ int kbins[kBins];
   __shared__ int scratch[kSchedThreads];
   __shared__ long long carry_run;
+  __shared__ int status;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = kSchedThreads / 64;
   for (int i = threadIdx.x; i < kBins; i += kSchedThreads) { qbins[i] = 0; kbins[i] = 0; }
-  if (threadIdx.x == 0) carry_run = 0;
+  if (threadIdx.x == 0) { carry_run = 0; status = kSchedOk; }
   __syncthreads();
 
-  // Pass 1: tiles per length class (class = number of query tiles of the sequence, saturating).
+  // Pass 1: tiles per length class (class = number of query tiles of the sequence, saturating).  Every entry of
+  // cu_seqlens is checked here; the checks are local (each end against its predecessor and the token count), and
+  // together they bound the tile counts and carry slots by what the caller's buffers were sized for.
   for (int s = threadIdx.x; s < p.num_seqs; s += kSchedThreads) {
     int start, len;
-    seq_bounds(p, s, &start, &len);
+    if (!seq_bounds(p, s, &start, &len)) status = kSchedBadCu;
     const int nq = (len + kBlockQ - 1) / kBlockQ, nk = (len + p.key_tile - 1) / p.key_tile;
     const int cls = min(nq, kBins - 1);
     if (nq) atomicAdd(&qbins[cls], nq);
     if (nk && p.want_key_tiles) atomicAdd(&kbins[cls], nk);
   }
   __syncthreads();
+  if (status != kSchedOk) {      // uniform: nothing is scheduled, every output row is zero-filled as uncovered
+    if (threadIdx.x == 0) { p.counts[kCountQ] = 0; p.counts[kCountK] = 0; p.counts[kCountStatus] = status; p.counts[kCountCovered] = 0; }
+    if (p.want_key_tiles)
+      for (int h = threadIdx.x; h < p.num_heads; h += kSchedThreads) p.head_queue[h] = 0;
+    return;
+  }
   descending_offsets(qbins, scratch);
   if (p.want_key_tiles) descending_offsets(kbins, scratch);
 
@@ -96,6 +99,12 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
       __syncthreads();
       if (threadIdx.x == kSchedThreads - 1) carry_run = base + sc[threadIdx.x];
       __syncthreads();
+    }
+    if (carry_run > p.carry_capacity) {      // uniform: the caller's max_seqlen (or slot count) was too small
+      if (threadIdx.x == 0) { p.counts[kCountQ] = 0; p.counts[kCountK] = 0; p.counts[kCountStatus] = kSchedCarryOverflow; p.counts[kCountCovered] = 0; }
+      if (p.want_key_tiles)
+        for (int h = threadIdx.x; h < p.num_heads; h += kSchedThreads) p.head_queue[h] = 0;
+      return;
     }
   }
   __syncthreads();
@@ -128,8 +137,12 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
   __syncthreads();
   // After the scatter, the lightest bin (work 0) ends at the total count.
   if (threadIdx.x == 0) {
-    p.counts[0] = qbins[0];
-    p.counts[1] = p.want_key_tiles ? kbins[0] : 0;
+    p.counts[kCountQ] = qbins[0];
+    p.counts[kCountK] = p.want_key_tiles ? kbins[0] : 0;
+    p.counts[kCountStatus] = kSchedOk;
+    int start = 0, len = (int)p.total_tokens;      // fixed-length mode: every row belongs to a sequence
+    if (p.cu != nullptr) seq_bounds(p, p.num_seqs - 1, &start, &len);
+    p.counts[kCountCovered] = start + len;
   }
   if (p.want_key_tiles)
     for (int h = threadIdx.x; h < p.num_heads; h += kSchedThreads) p.head_queue[h] = 0;

@@ -6,6 +6,7 @@ been built, or a call reports an error, the operators raise.
 from __future__ import annotations
 
 import ctypes
+import math
 import os
 from typing import Optional
 
@@ -14,7 +15,7 @@ import torch
 from .utils import custom_op
 
 _LIB_NAME = "libsba.so"
-ABI_VERSION = 2          # SBA_VERSION of include/sba.h this binding mirrors
+ABI_VERSION = 3          # SBA_VERSION of include/sba.h this binding mirrors
 _lib = None
 # Optional ctypes array of hipEvent_t handed to the next calls as SbaArgs.trace_events (benchmarks only).
 TRACE_EVENTS = None
@@ -43,11 +44,21 @@ class SbaArgs(ctypes.Structure):
         ("d_o", SbaTensor), ("d_rem", SbaVector), ("dq", SbaTensor), ("dk", SbaTensor), ("dv", SbaTensor),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t), ("stream", ctypes.c_void_p),
         ("trace_events", ctypes.POINTER(ctypes.c_void_p)),
-        ("add_remainder", ctypes.c_int32), ("reserved0", ctypes.c_int32),
+        ("add_remainder", ctypes.c_int32), ("reserved0", ctypes.c_int32), ("carry_slots", ctypes.c_int64),
     ]
 
 
-EXPORTS = ("sba_version", "sba_strerror", "sba_workspace_bytes", "sba_fwd", "sba_bwd")
+class SbaPlan(ctypes.Structure):
+    _fields_ = [("status", ctypes.c_int32), ("longest", ctypes.c_int32), ("covered_tokens", ctypes.c_int64),
+                ("query_tiles", ctypes.c_int64), ("key_tiles", ctypes.c_int64), ("carry_slots", ctypes.c_int64),
+                ("pairs", ctypes.c_int64)]
+
+
+EXPORTS = ("sba_version", "sba_strerror", "sba_workspace_bytes", "sba_plan_host", "sba_fwd", "sba_bwd")
+STATUS_OFFSET = 8        # SBA_STATUS_OFFSET: the scheduler's status word inside the workspace
+# Debugging aid for the tests: fill the carry buffer and the workspaces with NaN bit patterns before every launch,
+# so that a kernel reading a slot nobody wrote shows up as NaN instead of passing on whatever the allocator returned.
+POISON = os.environ.get("SBA_DEBUG_POISON", "0") == "1"
 
 
 def library_path() -> str:
@@ -68,6 +79,8 @@ def lib():
         handle.sba_strerror.argtypes = [ctypes.c_int]
         handle.sba_workspace_bytes.restype = ctypes.c_int
         handle.sba_workspace_bytes.argtypes = [ctypes.POINTER(SbaArgs)] + [ctypes.POINTER(ctypes.c_size_t)] * 3
+        handle.sba_plan_host.restype = ctypes.c_int
+        handle.sba_plan_host.argtypes = [ctypes.POINTER(SbaArgs), ctypes.c_void_p, ctypes.POINTER(SbaPlan)]
         for name in ("sba_fwd", "sba_bwd"):
             fn = getattr(handle, name)
             fn.restype = ctypes.c_int
@@ -110,7 +123,31 @@ def _require_gpu(*tensors):
             raise RuntimeError("stick-breaking attention runs on the GPU only (got a CPU tensor); there is no CPU path")
 
 
-def _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current) -> SbaArgs:
+def plan_host(cu_seqlens_host: Optional[torch.Tensor], cu_has_leading_zero: bool, total_tokens: int,
+              num_seqs: Optional[int] = None, attend_current: bool = False) -> SbaPlan:
+    """What the device scheduler will derive from ``cu_seqlens``, computed by the library on the host from a host
+    copy (sba_plan_host): validity, tile counts, the exact number of carry slots per head, visible pairs."""
+    a = SbaArgs()
+    a.total_tokens = int(total_tokens)
+    a.attend_current = 1 if attend_current else 0
+    ptr = None
+    if cu_seqlens_host is not None:
+        assert cu_seqlens_host.device.type == "cpu"
+        if cu_seqlens_host.dtype not in (torch.int32, torch.int64):
+            cu_seqlens_host = cu_seqlens_host.to(torch.int64)
+        cu_seqlens_host = cu_seqlens_host.contiguous()
+        a.num_seqs = cu_seqlens_host.numel() - (1 if cu_has_leading_zero else 0)
+        a.cu_is_int64 = 1 if cu_seqlens_host.dtype == torch.int64 else 0
+        a.cu_has_leading_zero = 1 if cu_has_leading_zero else 0
+        ptr = cu_seqlens_host.data_ptr()
+    else:
+        a.num_seqs = int(num_seqs)
+    out = SbaPlan()
+    _check(lib().sba_plan_host(ctypes.byref(a), ptr, ctypes.byref(out)), "sba_plan_host")
+    return out
+
+
+def _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, carry_slots=0) -> SbaArgs:
     if q.dtype not in _DTYPES:
         raise TypeError(f"unsupported dtype {q.dtype}")
     a = SbaArgs()
@@ -128,6 +165,7 @@ def _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, atte
         a.cu_is_int64 = 1 if cu_seqlens.dtype == torch.int64 else 0
         a.cu_has_leading_zero = 1 if cu_has_leading_zero else 0
     a.max_seqlen = int(max_seqlen) if max_seqlen else 0
+    a.carry_slots = int(carry_slots) if (carry_slots and not fixed) else 0
     a.logit_scale = float(logit_scale)
     a.attend_current = 1 if attend_current else 0
     a.stream = torch.cuda.current_stream(q.device).cuda_stream
@@ -144,14 +182,17 @@ def prepare_cu_seqlens(cu_seqlens: torch.Tensor, device) -> torch.Tensor:
     return cu_seqlens.contiguous()
 
 
-def carry_elems(num_heads: int, total_tokens: int, num_seqs: int, max_seqlen, fixed: bool) -> int:
-    """fp32 elements of the ``carry`` buffer the forward fills for the backward: the same bound the library
-    reports through ``sba_workspace_bytes`` (one value per query row and 32-key sub-tile the row sweeps),
-    computed here from shapes alone so that it can be traced by torch.compile."""
+def carry_elems(num_heads: int, total_tokens: int, num_seqs: int, max_seqlen, fixed: bool, carry_slots: int = 0) -> int:
+    """fp32 elements of the ``carry`` buffer the forward fills for the backward: what the library reports
+    through ``sba_workspace_bytes`` (one value per query row and 32-key sub-tile the row sweeps), computed
+    here from shapes alone so that it can be traced by torch.compile.  ``carry_slots`` > 0 is the exact
+    per-head count from ``plan_host``; otherwise packed batches use the bound T * max_seqlen / 64."""
     T, B = total_tokens, num_seqs
     if fixed:
         m = -(-T // 128)
         slots = B * 256 * m * (m + 1)
+    elif carry_slots:
+        slots = carry_slots
     else:
         max_len = max_seqlen if (max_seqlen and 0 < max_seqlen < T) else T
         slots = -(-(T * max_len) // 64) + 6 * T + 512 * B
@@ -159,11 +200,15 @@ def carry_elems(num_heads: int, total_tokens: int, num_seqs: int, max_seqlen, fi
     return nbytes // 4
 
 
-def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, add_remainder, o, rem,
-                neg_log_acc, carry):
+def _poison(t: torch.Tensor):
+    t.view(torch.uint8).fill_(0xFF)          # every fp32 / 16-bit word becomes a NaN pattern, every int32 becomes -1
+
+
+def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, carry_slots, logit_scale, attend_current, add_remainder,
+                o, rem, neg_log_acc, carry):
     fixed = cu_seqlens is None
     with torch.cuda.device(q.device):
-        a = _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current)
+        a = _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, carry_slots)
         a.add_remainder = 1 if add_remainder else 0
         a.q, a.k, a.v, a.o = (_tensor(t, fixed) for t in (q, k, v, o))
         a.rem = _vector(rem, fixed)
@@ -172,6 +217,10 @@ def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scal
         _check(lib().sba_workspace_bytes(ctypes.byref(a), ctypes.byref(need), None, ctypes.byref(need_carry)), "sba_workspace_bytes")
         ws = torch.empty(need.value, dtype=torch.uint8, device=q.device)
         a.workspace, a.workspace_bytes = ws.data_ptr(), need.value
+        if POISON:
+            _poison(ws)
+            if carry.numel() > 0:
+                _poison(carry)
         if carry.numel() > 0:
             if carry.numel() * 4 < need_carry.value:
                 raise RuntimeError(f"carry buffer too small: {carry.numel() * 4} < {need_carry.value} bytes")
@@ -179,11 +228,11 @@ def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scal
         _check(lib().sba_fwd(ctypes.byref(a)), "sba_fwd")
 
 
-def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current,
-                add_remainder, dq, dk, dv):
+def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leading_zero, max_seqlen, carry_slots, logit_scale,
+                attend_current, add_remainder, dq, dk, dv):
     fixed = cu_seqlens is None
     with torch.cuda.device(q.device):
-        a = _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current)
+        a = _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, carry_slots)
         a.add_remainder = 1 if add_remainder else 0
         a.row_stat = neg_log_acc.data_ptr() if neg_log_acc.numel() > 0 else None
         a.q, a.k, a.v, a.d_o, a.dq, a.dk, a.dv = (_tensor(t, fixed) for t in (q, k, v, do, dq, dk, dv))
@@ -193,6 +242,8 @@ def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leadin
         _check(lib().sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(need), None), "sba_workspace_bytes")
         ws = torch.empty(need.value, dtype=torch.uint8, device=q.device)
         a.workspace, a.workspace_bytes = ws.data_ptr(), need.value
+        if POISON:
+            _poison(ws)
         _check(lib().sba_bwd(ctypes.byref(a)), "sba_bwd")
 
 
@@ -202,44 +253,53 @@ def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leadin
 # only".
 @custom_op("varlen_fwd", mutates_args={"o", "rem", "neg_log_acc", "carry"})
 def varlen_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor, cu_has_leading_zero: bool,
-               max_seqlens: int, logit_scale: float, attend_current: bool, add_remainder: bool, o: torch.Tensor,
-               rem: torch.Tensor, neg_log_acc: torch.Tensor, carry: torch.Tensor) -> None:
-    _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlens, logit_scale, attend_current, add_remainder, o, rem,
-                neg_log_acc, carry)
+               max_seqlens: int, carry_slots: int, logit_scale: float, attend_current: bool, add_remainder: bool,
+               o: torch.Tensor, rem: torch.Tensor, neg_log_acc: torch.Tensor, carry: torch.Tensor) -> None:
+    _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlens, carry_slots, logit_scale, attend_current, add_remainder,
+                o, rem, neg_log_acc, carry)
 
 
 @custom_op("varlen_bwd", mutates_args={"dq", "dk", "dv"})
 def varlen_bwd(do: torch.Tensor, drem: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, carry: torch.Tensor,
                neg_log_acc: torch.Tensor, cu_seqlens: torch.Tensor, cu_has_leading_zero: bool, max_seqlens: int,
-               logit_scale: float, attend_current: bool, add_remainder: bool, dq: torch.Tensor, dk: torch.Tensor,
-               dv: torch.Tensor) -> None:
-    _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leading_zero, max_seqlens, logit_scale, attend_current,
-                add_remainder, dq, dk, dv)
+               carry_slots: int, logit_scale: float, attend_current: bool, add_remainder: bool, dq: torch.Tensor,
+               dk: torch.Tensor, dv: torch.Tensor) -> None:
+    _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leading_zero, max_seqlens, carry_slots, logit_scale,
+                attend_current, add_remainder, dq, dk, dv)
 
 
 @custom_op("attn_fwd", mutates_args={"o", "rem", "neg_log_acc", "carry"})
 def attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_scale: float, attend_current: bool, add_remainder: bool,
              o: torch.Tensor, rem: torch.Tensor, neg_log_acc: torch.Tensor, carry: torch.Tensor) -> None:
-    _launch_fwd(q, k, v, None, False, q.size(2), logit_scale, attend_current, add_remainder, o, rem, neg_log_acc, carry)
+    _launch_fwd(q, k, v, None, False, q.size(2), 0, logit_scale, attend_current, add_remainder, o, rem, neg_log_acc, carry)
 
 
 @custom_op("attn_bwd", mutates_args={"dq", "dk", "dv"})
 def attn_bwd(do: torch.Tensor, drem: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, carry: torch.Tensor,
              neg_log_acc: torch.Tensor, logit_scale: float, attend_current: bool, add_remainder: bool, dq: torch.Tensor,
              dk: torch.Tensor, dv: torch.Tensor) -> None:
-    _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, None, False, q.size(2), logit_scale, attend_current, add_remainder,
+    _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, None, False, q.size(2), 0, logit_scale, attend_current, add_remainder,
                 dq, dk, dv)
 
 
-def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, want_carry, add_remainder=False):
+def _same_dtype(q, **others):
+    for name, t in others.items():
+        if t is not None and t.dtype != q.dtype:
+            raise TypeError(f"{name} has dtype {t.dtype}, q has {q.dtype}: q, k, v and the gradients must share one dtype")
+
+
+def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current, want_carry, add_remainder=False,
+            carry_slots=0):
     """Launch the forward.  Returns (o, rem, row_stat, carry or None).  Packed mode when cu_seqlens is given.
     ``carry`` is the buffer the backward needs; it is only produced when ``want_carry``.  With ``add_remainder`` the
-    first output is ``o + rem[..., None] * v``."""
+    first output is ``o + rem[..., None] * v``.  ``carry_slots``: exact per-head size of ``carry`` from ``plan_host``
+    (0 = the bound derived from ``max_seqlen``); the backward must be given the same value."""
     _require_gpu(q, k, v)
     fixed = cu_seqlens is None
     q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)
     if q.dtype not in _DTYPES:
         raise TypeError(f"unsupported dtype {q.dtype}")
+    _same_dtype(q, k=k, v=v)
     o = torch.empty_like(q)
     if o.stride(-1) != 1:
         o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
@@ -250,22 +310,24 @@ def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, a
         if fixed:
             n_carry = carry_elems(q.size(1), q.size(2), q.size(0), None, True)
         else:
-            n_carry = carry_elems(q.size(0), q.size(1), cu_seqlens.numel() - (1 if cu_has_leading_zero else 0), max_seqlen, False)
+            n_carry = carry_elems(q.size(0), q.size(1), cu_seqlens.numel() - (1 if cu_has_leading_zero else 0), max_seqlen, False,
+                                  int(carry_slots))
     carry = torch.empty(n_carry, dtype=torch.float32, device=q.device)
     if fixed:
         attn_fwd(q, k, v, float(logit_scale), bool(attend_current), bool(add_remainder), o, rem, row_stat, carry)
     else:
-        varlen_fwd(q, k, v, cu_seqlens, bool(cu_has_leading_zero), int(max_seqlen) if max_seqlen else 0, float(logit_scale),
-                   bool(attend_current), bool(add_remainder), o, rem, row_stat, carry)
+        varlen_fwd(q, k, v, cu_seqlens, bool(cu_has_leading_zero), int(max_seqlen) if max_seqlen else 0, int(carry_slots),
+                   float(logit_scale), bool(attend_current), bool(add_remainder), o, rem, row_stat, carry)
     return o, rem, row_stat, (carry if want_carry else None)
 
 
 def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current,
-             row_stat=None, add_remainder=False):
+             row_stat=None, add_remainder=False, carry_slots=0):
     """Launch the backward.  Returns (dq, dk, dv).  ``row_stat`` (the forward's third output) is needed when the
-    forward ran with ``add_remainder``."""
+    forward ran with ``add_remainder``.  Rows of a packed batch that belong to no sequence get zero gradients."""
     _require_gpu(q, k, v, do, drem, carry)
     fixed = cu_seqlens is None
+    _same_dtype(q, k=k, v=v, do=do)
     do = rows_contiguous(do)
     q, k, v = rows_contiguous(q), rows_contiguous(k), rows_contiguous(v)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
@@ -281,5 +343,6 @@ def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seql
         attn_bwd(do, drem, q, k, v, carry, row_stat, float(logit_scale), bool(attend_current), bool(add_remainder), dq, dk, dv)
     else:
         varlen_bwd(do, drem, q, k, v, carry, row_stat, cu_seqlens, bool(cu_has_leading_zero),
-                   int(max_seqlen) if max_seqlen else 0, float(logit_scale), bool(attend_current), bool(add_remainder), dq, dk, dv)
+                   int(max_seqlen) if max_seqlen else 0, int(carry_slots), float(logit_scale), bool(attend_current),
+                   bool(add_remainder), dq, dk, dv)
     return dq, dk, dv

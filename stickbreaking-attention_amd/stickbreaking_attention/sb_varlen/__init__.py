@@ -18,10 +18,13 @@ class StickBreakingAttention(torch.autograd.Function):
     ``zero_start`` was requested; the scheduler kernel skips it instead of the host slicing the tensor."""
 
     @staticmethod
-    def forward(ctx, q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current, leading_zero=False, add_remainder=False):
+    def forward(ctx, q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current, leading_zero=False, add_remainder=False,
+                carry_slots=0):
         need_grad = any(ctx.needs_input_grad[:3])
         o, rem, row_stat, carry = _native.forward(q, k, v, cu_seqlens, leading_zero, max_seqlens, inv_temp,
-                                                 attend_current, want_carry=need_grad, add_remainder=add_remainder)
+                                                 attend_current, want_carry=need_grad, add_remainder=add_remainder,
+                                                 carry_slots=carry_slots)
+        ctx.carry_slots = carry_slots
         ctx.save_for_backward(q, k, v, carry, cu_seqlens, row_stat if add_remainder else None)
         ctx.add_remainder = add_remainder
         ctx.logit_scale = inv_temp
@@ -35,22 +38,35 @@ class StickBreakingAttention(torch.autograd.Function):
         q, k, v, carry, cu_seqlens, row_stat = ctx.saved_tensors
         dq, dk, dv = _native.backward(do, drem, q, k, v, carry, cu_seqlens, ctx.leading_zero,
                                       ctx.max_seqlens, ctx.logit_scale, ctx.attend_current,
-                                      row_stat=row_stat, add_remainder=ctx.add_remainder)
-        return dq, dk, dv, None, None, None, None, None, None
+                                      row_stat=row_stat, add_remainder=ctx.add_remainder, carry_slots=ctx.carry_slots)
+        return dq, dk, dv, None, None, None, None, None, None, None
 
 
 def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, zero_start=True, attend_current=False,
                    add_remainder=False):
     """``add_remainder=True`` returns ``(o + rem[..., None] * v, rem)``: the combination every caller of the
     reference forms from its outputs (tests/test_varlen.py:103), fused into the kernels' epilogues."""
-    cu_seqlens = _native.prepare_cu_seqlens(cu_seqlens, q.device)
+    # The lengths are on the host when cu_seqlens was given as a CPU tensor, or after the one device-to-host copy that
+    # stands in for the reference's `assert cu_seqlens[0] == 0` (sb_varlen/__init__.py:71-73, the same host sync).
+    # They are then validated there and the carry buffer is sized exactly; a device-only cu_seqlens is validated by
+    # the scheduler kernel and the buffer is sized from the bound total_tokens * max_seqlens / 64.
+    cu_host = cu_seqlens if cu_seqlens.device.type == "cpu" else None
     if zero_start:
-        assert cu_seqlens[0] == 0          # same check (and host sync) as sb_varlen/__init__.py:71-73
+        if cu_host is None and not torch.compiler.is_compiling():
+            cu_host = cu_seqlens.cpu()
+        assert (cu_host if cu_host is not None else cu_seqlens)[0] == 0
     _native._require_gpu(q, k, v)
+    carry_slots = 0
+    if cu_host is not None:
+        plan = _native.plan_host(cu_host, bool(zero_start), q.size(1))
+        if plan.status != 0:
+            raise ValueError("cu_seqlens must be non-decreasing sequence ends within [0, total_tokens]")
+        carry_slots = int(plan.carry_slots)
+    cu_seqlens = _native.prepare_cu_seqlens(cu_seqlens, q.device)
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
     return StickBreakingAttention.apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current, bool(zero_start),
-                                        bool(add_remainder))
+                                        bool(add_remainder), carry_slots)
 
 
 def sb_attn_varlen_(q, k, v, inv_temp, cu_seqlens, max_seqlens, attend_current):

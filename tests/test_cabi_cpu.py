@@ -29,11 +29,12 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol(native):
     names = declared_functions()
-    assert set(names) == set(native.EXPORTS) == {"sba_version", "sba_strerror", "sba_workspace_bytes", "sba_fwd", "sba_bwd"}
+    assert set(names) == set(native.EXPORTS) == {"sba_version", "sba_strerror", "sba_workspace_bytes", "sba_plan_host", "sba_fwd",
+                                                 "sba_bwd"}
     lib = native.lib()
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.sba_version() == native.ABI_VERSION == 2
+    assert lib.sba_version() == native.ABI_VERSION == 3
     assert lib.sba_strerror(0) == b"ok"
     for code in range(-8, 0):
         assert lib.sba_strerror(code) not in (b"ok", b"unknown status")
@@ -42,16 +43,19 @@ def test_library_exports_every_declared_symbol(native):
 
 def test_struct_layout_matches_header(native, tmp_path):
     src = tmp_path / "sz.c"
-    src.write_text('#include "sba.h"\n#include <stdio.h>\n#include <stddef.h>\nint main(){printf("%zu %zu %zu %zu %zu %zu\\n", '
+    src.write_text('#include "sba.h"\n#include <stdio.h>\n#include <stddef.h>\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu\\n", '
                    "sizeof(SbaArgs), offsetof(SbaArgs,q), offsetof(SbaArgs,carry), offsetof(SbaArgs,d_o), "
-                   "offsetof(SbaArgs,workspace), offsetof(SbaArgs,trace_events));}\n")
+                   "offsetof(SbaArgs,workspace), offsetof(SbaArgs,trace_events), offsetof(SbaArgs,carry_slots), "
+                   "sizeof(SbaPlan), offsetof(SbaPlan,pairs));}\n")
     exe = tmp_path / "sz"
     import subprocess
 
     subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
     got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
     A = native.SbaArgs
-    assert got == [ctypes.sizeof(A), A.q.offset, A.carry.offset, A.d_o.offset, A.workspace.offset, A.trace_events.offset]
+    P = native.SbaPlan
+    assert got == [ctypes.sizeof(A), A.q.offset, A.carry.offset, A.d_o.offset, A.workspace.offset, A.trace_events.offset,
+                   A.carry_slots.offset, ctypes.sizeof(P), P.pairs.offset]
 
 
 def _args(native, H, D, T, B, varlen=True, max_seqlen=0, dtype=0):
@@ -99,6 +103,75 @@ def test_python_carry_size_matches_library(native):
         a = _args(native, H, 64, T, B, varlen=False)
         assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, ctypes.byref(carry)) == 0
         assert native.carry_elems(H, T, B, None, True) * 4 == carry.value
+
+
+def test_exact_carry_slots_shrink_the_buffers(native):
+    """With the exact per-head slot count from the host plan the carry buffer (and the backward's prefix plane) are the
+    need itself, not the total_tokens * max_seqlen / 64 bound: the adversarial batch (2048 short sequences and one of
+    16384) drops from about 4.5x the need to 1.0x."""
+    import bench
+
+    lib = native.lib()
+    lengths = bench.lengths_for("c5")
+    T, H = sum(lengths), 32
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int32)
+    plan = native.plan_host(cu, True, T)
+    exact = sum(256 * m * (m + 1) for m in (-(-n // 128) for n in lengths))
+    assert plan.status == 0 and plan.carry_slots == exact and plan.longest == 16384 and plan.covered_tokens == T
+    assert plan.query_tiles == sum(-(-n // 128) for n in lengths) and plan.key_tiles == sum(-(-n // 64) for n in lengths)
+    assert plan.pairs == sum(n * (n - 1) // 2 for n in lengths)
+    carry_bound, carry_exact, bwd_exact = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    a = _args(native, H, 128, T, len(lengths), max_seqlen=16384)
+    assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, ctypes.byref(carry_bound)) == 0
+    a.carry_slots = plan.carry_slots
+    assert lib.sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(bwd_exact), ctypes.byref(carry_exact)) == 0
+    need = exact * H * 4
+    assert need <= carry_exact.value <= need + 256 and carry_bound.value > 4 * need
+    assert bwd_exact.value <= 1.2 * need + (1 << 22)          # prefix plane + tile lists + per-row scalars
+    assert native.carry_elems(H, T, len(lengths), 16384, False, exact) * 4 == carry_exact.value
+    a.carry_slots = -1
+    assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, None) == -6
+    a.carry_slots, a.reserved0 = 0, 1
+    assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, None) == -6
+
+
+def test_host_plan_rejects_what_the_scheduler_rejects(native):
+    """sba_plan_host runs the scheduler's own reading of cu_seqlens (one shared function) on a host copy: decreasing
+    ends, ends beyond total_tokens, negative entries and a leading entry other than 0 void the schedule; empty
+    sequences and trailing uncovered tokens are fine."""
+    T = 100
+    good = [
+        ([10, 10, 40, 100], False, 100), ([0, 10, 40], True, 40), ([100], False, 100), ([0, 0, 0], False, 0),
+        ([5], False, 5), ([0, 100], True, 100),
+    ]
+    for cu, lead, covered in good:
+        for dt in (torch.int32, torch.int64):
+            plan = native.plan_host(torch.tensor(cu, dtype=dt), lead, T)
+            assert plan.status == 0 and plan.covered_tokens == covered, (cu, lead)
+    bad = [([10, 5, 40], False), ([10, 101], False), ([-1, 10], False), ([3, 10], True), ([0, 50, 20], True),
+           ([2 ** 40, 2 ** 40 + 1], False), ([10, -2 ** 31], False)]
+    for cu, lead in bad:
+        plan = native.plan_host(torch.tensor(cu, dtype=torch.int64), lead, T)
+        assert plan.status == 1 and plan.query_tiles == 0 and plan.key_tiles == 0 and plan.carry_slots == 0, (cu, lead)
+    # for every valid batch the tile counts stay inside what sba_workspace_bytes reserves from shapes alone
+    rng = np.random.default_rng(5)
+    for _ in range(300):
+        B = int(rng.integers(1, 60))
+        lengths = rng.integers(0, int(rng.choice([3, 70, 300, 3000])), size=B)
+        pad = int(rng.integers(0, 200))
+        total = int(lengths.sum()) + pad
+        if total == 0:
+            continue
+        plan = native.plan_host(torch.tensor(np.cumsum(lengths)), False, total)
+        assert plan.status == 0 and plan.covered_tokens == int(lengths.sum())
+        assert plan.query_tiles <= -(-total // 128) + B and plan.key_tiles <= -(-total // 64) + B
+        idle = -(-total // 128) + B - plan.query_tiles          # workgroups left to zero-fill the uncovered rows
+        assert idle * 128 >= pad
+        mx = max(int(lengths.max()), 1)
+        assert plan.carry_slots <= -(-(total * mx) // 64) + 6 * total + 512 * B
+    # fixed-length mode
+    a = native.plan_host(None, False, 500, num_seqs=4)
+    assert a.status == 0 and a.query_tiles == 16 and a.carry_slots == 4 * 256 * 4 * 5 and a.pairs == 4 * 500 * 499 // 2
 
 
 def test_custom_ops_are_registered(native):

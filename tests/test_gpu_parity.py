@@ -6,10 +6,15 @@ in fp32/fp64 on the same bf16-rounded inputs.  A bf16 output cannot be closer to
 in the last place, which exceeds 2e-2 once |value| >= 4, so where |reference| is that large the bound is one bf16
 ulp of the reference (2^-7 |ref|) instead.  For fp32 inputs the bar is 1e-4.
 
+Every check prints, per tensor, the max-abs error, how many elements exceed the bound, the largest excess and
+|reference| at the worst element.
+
 The adversarial configuration scales q and k by 3.  dq and dk are contractions of the 16-bit-rounded logit
-gradient against k and q (the reference rounds at the same point: sb_varlen_bwd.py:449-451), so their rounding
-noise grows with the operand magnitude; for those two tensors of that configuration the absolute part of the
-bound is scaled by the same factor 3 (6e-2), and the measured errors are printed.
+gradient against k and q (the reference rounds at the same point: sb_varlen_bwd.py:449-450); with |dZ| up to 16
+and |k| ~ 3 that rounding alone puts a handful of elements a few thousandths beyond the bound.  That floor is not
+fitted: the test evaluates `oracle.rounding_floor` (float64 arithmetic, P and dZ rounded to bf16 before their
+contractions, bf16 outputs) on the same inputs and allows the kernels the floor's own largest excess plus 2e-3 for
+the fp32 arithmetic in between.
 """
 import math
 
@@ -25,21 +30,29 @@ pytestmark = pytest.mark.gpu
 NAMES = ["o", "rem", "dq", "dk", "dv"]
 
 
-def tol_check(name, got, ref, dtype, label, operand_scale=1.0):
+def error_bound(ref, dtype):
+    if dtype == torch.float32:
+        return torch.full_like(ref, 1e-4)
+    if dtype == torch.float16:
+        return torch.maximum(torch.full_like(ref, 2e-2), ref.abs() * 2.0 ** -10)
+    return torch.maximum(torch.full_like(ref, 2e-2), ref.abs() * 2.0 ** -7)
+
+
+def tol_check(name, got, ref, dtype, label, allowed_excess=0.0):
+    """Asserts |got - ref| <= bound (+ allowed_excess, which only the adversarial configuration uses and derives
+    from the rounding floor).  Returns the largest excess over the bound (negative when inside)."""
     got = got.detach().double().cpu()
     ref = ref.double()
     assert not torch.isnan(got).any(), f"{label}: NaN in {name}"
     err = (got - ref).abs()
-    if dtype == torch.float32:
-        bound = torch.full_like(ref, 1e-4)
-    elif dtype == torch.float16:
-        bound = torch.maximum(torch.full_like(ref, 2e-2), ref.abs() * 2.0 ** -10)
-    else:
-        absolute = 2e-2 * (operand_scale if name in ("dq", "dk") else 1.0)
-        bound = torch.maximum(torch.full_like(ref, absolute), ref.abs() * 2.0 ** -7)
-    worst = (err - bound).max().item()
-    print(f"{label} {name}: max-abs err {err.max().item():.3e} (ref max {ref.abs().max().item():.2f})", flush=True)
-    assert worst <= 0, f"{label}: {name} max-abs err {err.max().item():.4e} exceeds tolerance by {worst:.3e}"
+    excess = err - error_bound(ref, dtype)
+    worst = excess.max().item() if excess.numel() else 0.0
+    at = int(excess.argmax()) if excess.numel() else 0
+    print(f"{label} {name}: max-abs err {err.max().item() if err.numel() else 0:.3e}, {int((excess > 0).sum())} of {excess.numel()} "
+          f"beyond the bound, largest excess {worst:.3e} at |ref| = {ref.flatten()[at].abs().item() if excess.numel() else 0:.3f} "
+          f"(ref max {ref.abs().max().item() if ref.numel() else 0:.2f})", flush=True)
+    assert worst <= allowed_excess, f"{label}: {name} exceeds the bound by {worst:.3e} (allowed {allowed_excess:.3e})"
+    return worst
 
 
 def run_varlen(q, k, v, cu, lengths, zero_start, attend_current, do, drem, scale=None, max_seqlens=True):
@@ -266,7 +279,14 @@ def test_config2_forward_full_size(gpu_device):
 
 
 def test_config3_full_size(gpu_device):
-    inp, got = _full_size("c3", gpu_device, [0, 17, 31])
+    # six of the 32 heads against the oracle, drawn from a seed that changes from day to day and is printed, so
+    # that over time every head gets checked; heads 0 and 31 (first / last XCD) are always among them
+    import datetime
+
+    seed = datetime.date.today().toordinal()
+    heads = sorted({0, 31} | set(int(h) for h in np.random.default_rng(seed).choice(np.arange(1, 31), 4, replace=False)))
+    print(f"c3: oracle heads {heads} (seed {seed})", flush=True)
+    inp, got = _full_size("c3", gpu_device, heads)
     # size-independent property over ALL heads: each sequence on its own (fixed-length entry point) reproduces
     # its slice of the packed result bit for bit
     from stickbreaking_attention import sb_attn
@@ -300,27 +320,45 @@ def test_config4_fixed_full_size(gpu_device):
             tol_check(n, a[b:b + 1, h:h + 1], r, torch.bfloat16, f"c4[{b},{h}]")
 
 
-def test_config5_adversarial_ragged(gpu_device):
-    # 2048 sequences of 1..64 tokens plus one of 16384, zero_start=True, saturating logits.
-    # The oracle covers every short sequence on two heads and the long sequence on one head.
+def _check_against_floor(label, got, floor, exact):
+    """The adversarial configuration's bar: max(2e-2, 2^-7 |ref|) plus the largest excess that exact arithmetic with
+    bf16 matrix operands and bf16 outputs (`oracle.rounding_floor`) shows on the same inputs, plus 2e-3 for the fp32
+    arithmetic in between."""
+    for n, a, f, b in zip(NAMES, got, floor, exact):
+        floor_excess = ((f - b).abs() - error_bound(b, torch.bfloat16)).max().item()
+        print(f"{label} {n}: rounding floor max-abs err {(f - b).abs().max().item():.3e}, largest excess {floor_excess:.3e}", flush=True)
+        tol_check(n, a, b, torch.bfloat16, label, allowed_excess=max(floor_excess, 0.0) + 2e-3)
+
+
+@pytest.fixture(scope="module")
+def config5_run(gpu_device):
+    # 2048 sequences of 1..64 tokens plus one of 16384, zero_start=True, saturating logits (q, k ~ N(0, 9)).
     inp = bench.make_inputs("c5", gpu_device)
-    lengths = inp["lengths"]
-    got = run_varlen(inp["q"], inp["k"], inp["v"], inp["cu"], lengths, True, False, inp["do"], inp["drem"])
+    got = run_varlen(inp["q"], inp["k"], inp["v"], inp["cu"], inp["lengths"], True, False, inp["do"], inp["drem"])
     for t in got:
         assert torch.isfinite(t.float()).all()
-    short_T = sum(lengths[:-1])
     host = [inp[n].cpu() for n in ("q", "k", "v", "do", "drem")]
+    return inp["lengths"], host, [t.detach().cpu() for t in got]
+
+
+def test_config5_adversarial_short_sequences(config5_run):
+    # every short sequence on two heads, float64 oracle
+    lengths, host, got = config5_run
+    short_T = sum(lengths[:-1])
     cu_short = torch.tensor(np.cumsum(lengths[:-1]))
     heads = [3, 30]
-    ref = orc.varlen_stream(*(t[:, :short_T] for t in host[:3]), cu_short, do=host[3][:, :short_T], drem=host[4][:, :short_T],
-                            dtype=torch.float32, heads=heads)
-    for n, a, b in zip(NAMES, got, ref):
-        tol_check(n, a[heads, :short_T], b[heads], torch.bfloat16, "c5 short sequences", operand_scale=3.0)
+    short = [t[heads, :short_T] for t in host]
+    floor, exact = orc.varlen_rounding_floor(*short[:3], cu_short, short[3], short[4])
+    _check_against_floor("c5 short sequences", [t[heads, :short_T] for t in got], floor, exact)
+
+
+def test_config5_adversarial_long_sequence(config5_run):
+    # the 16384-token sequence on one head, float64 oracle
+    lengths, host, got = config5_run
+    short_T = sum(lengths[:-1])
     h = 9
-    sl = [t[h:h + 1, short_T:] for t in host]
-    ref = orc.varlen_stream(sl[0], sl[1], sl[2], [lengths[-1]], do=sl[3], drem=sl[4], dtype=torch.float32)
-    for n, a, b in zip(NAMES, got, ref):
-        tol_check(n, a[h:h + 1, short_T:], b, torch.bfloat16, "c5 long sequence", operand_scale=3.0)
+    floor, exact = orc.rounding_floor(*(t[h, short_T:] for t in host), with_exact=True)
+    _check_against_floor("c5 long sequence", [t[h, short_T:] for t in got], floor, exact)
 
 
 def test_forward_without_grad_skips_carry(gpu_device):
