@@ -47,6 +47,9 @@ extern "C" {
 #define SBA_SCHED_BAD_CU_SEQLENS 1
 #define SBA_SCHED_CARRY_TOO_SMALL 2
 
+/* Size of the static device scratch behind sba_fwd_static. */
+#define SBA_STATIC_SCRATCH_BYTES ((size_t)1 << 20)
+
 typedef enum SbaDtype { SBA_BF16 = 0, SBA_F32 = 1, SBA_F16 = 2 } SbaDtype;
 
 typedef enum SbaStatus {
@@ -59,7 +62,8 @@ typedef enum SbaStatus {
   SBA_ERR_ALIGN = -5,       /* a tensor base pointer is not aligned to its element size */
   SBA_ERR_SHAPE = -6,       /* non-positive sizes, total_tokens > 2^30, or a reserved field that is not 0 */
   SBA_ERR_WORKSPACE = -7,   /* workspace missing, not 256-byte aligned, or smaller than sba_workspace_bytes reports */
-  SBA_ERR_LAUNCH = -8       /* the HIP runtime rejected a launch (hipGetLastError) */
+  SBA_ERR_LAUNCH = -8,      /* the HIP runtime rejected a launch (hipGetLastError) */
+  SBA_ERR_TOO_LARGE = -9    /* sba_fwd_static: the tile schedule does not fit the library's static scratch */
 } SbaStatus;
 
 /* One strided [batch,] head, token, head_dim tensor (strides in elements; head_dim stride is 1). */
@@ -169,6 +173,22 @@ int sba_plan_host(const SbaArgs* args, const void* cu_seqlens_host, SbaPlan* pla
  * (sb_varlen_fwd.py:280-294).
  */
 int sba_fwd(const SbaArgs* args);
+
+/*
+ * The forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the same kernels and results as sba_fwd, with the tile schedule
+ * kept in a static device array of the library (SBA_STATIC_SCRATCH_BYTES = 1 MiB per GPU, held until the
+ * process ends) instead of a caller workspace.  args->workspace and args->workspace_bytes are ignored; all
+ * other buffers (inputs, o, rem, row_stat and, when a backward will follow, carry) are still the caller's.
+ * The call allocates nothing and frees nothing.  It returns SBA_ERR_TOO_LARGE when the forward workspace that
+ * sba_workspace_bytes reports exceeds the array (roughly total_tokens / 128 + num_seqs > 32000 query tiles).
+ * Every call on one GPU shares that GPU's array and rewrites all of it that it reads, so calls need not clear
+ * it, but two calls that overlap in time on one GPU (different streams or threads) race: order them.
+ * The scheduler status word is not readable by the caller here.
+ * No counterpart in the reference, whose launcher allocates its outputs and lock buffers on every call
+ * (sb_varlen_fwd.py:417-424, sb_varlen_bwd.py:569-572).
+ */
+int sba_fwd_static(const SbaArgs* args);
 
 /*
  * Backward: fills dq, dk, dv from q, k, v, carry, d_o, d_rem (and row_stat when add_remainder is set).

@@ -1,6 +1,8 @@
 // C ABI of libsba: argument validation, workspace layout and kernel launches.  See include/sba.h.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "../../include/sba.h"
 #include "sba_params.hpp"
 
@@ -86,8 +88,7 @@ int check_tensor(const SbaTensor& t, bool required, bool fixed) {
 sba::TensorRef ref(const SbaTensor& t, bool fixed) { return sba::TensorRef{t.ptr, fixed ? t.stride_batch : 0, t.stride_head, t.stride_token}; }
 sba::VectorRef vref(const SbaVector& t, bool fixed) { return sba::VectorRef{t.ptr, fixed ? t.stride_batch : 0, t.stride_head, t.stride_token}; }
 
-int run_sched(const SbaArgs* a, const Layout& L, bool want_key_tiles, bool want_carry_base, int key_tile, hipStream_t stream) {
-  char* ws = (char*)a->workspace;
+int run_sched(const SbaArgs* a, char* ws, const Layout& L, bool want_key_tiles, bool want_carry_base, int key_tile, hipStream_t stream) {
   sba::SchedParams sp{};
   sp.cu = a->cu_seqlens;
   sp.cu_is_int64 = a->cu_is_int64;
@@ -126,6 +127,7 @@ const char* sba_strerror(int status) {
     case SBA_ERR_SHAPE: return "sizes must be positive (and total_tokens <= 2^30)";
     case SBA_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
     case SBA_ERR_LAUNCH: return "kernel launch failed";
+    case SBA_ERR_TOO_LARGE: return "the problem needs more scratch than the library's static array holds";
     default: return "unknown status";
   }
 }
@@ -166,8 +168,33 @@ int sba_plan_host(const SbaArgs* a, const void* cu_host, SbaPlan* out) {
   return SBA_OK;
 }
 
-int sba_fwd(const SbaArgs* a) {
-  if (!a) return SBA_ERR_NULL;
+}  // extern "C"
+
+namespace {
+
+// Scratch of sba_fwd_static: the forward's tile schedule (counts, query-tile list, per-sequence carry offsets) kept in
+// a device array of the library instead of a caller workspace.  Every GPU the library runs on holds its own copy
+// until the process ends.  Host code never uses the array's name as an address: the device address is looked up
+// once per device with hipGetSymbolAddress and that pointer is what the kernels receive.
+constexpr size_t kStaticScratchBytes = SBA_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+int static_scratch(char** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return SBA_ERR_LAUNCH;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return SBA_ERR_LAUNCH;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = (char*)ptr;
+  return SBA_OK;
+}
+
+// The forward on a given workspace (the caller's, or the library's static scratch).
+int fwd_on(const SbaArgs* a, char* ws, size_t ws_bytes, bool ws_is_static) {
   Layout L;
   int st = plan(a, &L);
   if (st != SBA_OK) return st;
@@ -179,11 +206,11 @@ int sba_fwd(const SbaArgs* a) {
   if (!a->rem.ptr || !a->row_stat) return SBA_ERR_NULL;
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->o})
     if (t->ptr && ((uintptr_t)t->ptr % es)) return SBA_ERR_ALIGN;
-  if (!a->workspace || ((uintptr_t)a->workspace & 255) || a->workspace_bytes < L.fwd_bytes) return SBA_ERR_WORKSPACE;
+  if (ws_is_static && ws_bytes < L.fwd_bytes) return SBA_ERR_TOO_LARGE;
+  if (!ws || ((uintptr_t)ws & 255) || ws_bytes < L.fwd_bytes) return SBA_ERR_WORKSPACE;
   hipStream_t stream = (hipStream_t)a->stream;
-  if ((st = run_sched(a, L, false, a->carry != nullptr, kBlockK, stream)) != SBA_OK) return st;
+  if ((st = run_sched(a, ws, L, false, a->carry != nullptr, kBlockK, stream)) != SBA_OK) return st;
 
-  char* ws = (char*)a->workspace;
   sba::FwdParams p{};
   p.q = ref(a->q, fixed); p.k = ref(a->k, fixed); p.v = ref(a->v, fixed); p.o = ref(a->o, fixed);
   p.rem = vref(a->rem, fixed);
@@ -213,6 +240,23 @@ int sba_fwd(const SbaArgs* a) {
   if (e != hipSuccess) return SBA_ERR_LAUNCH;
   if (ev && hipEventRecord(ev[1], stream) != hipSuccess) return SBA_ERR_LAUNCH;
   return SBA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sba_fwd(const SbaArgs* a) {
+  if (!a) return SBA_ERR_NULL;
+  return fwd_on(a, (char*)a->workspace, a->workspace_bytes, false);
+}
+
+int sba_fwd_static(const SbaArgs* a) {
+  if (!a) return SBA_ERR_NULL;
+  char* ws = nullptr;
+  const int st = static_scratch(&ws);
+  if (st != SBA_OK) return st;
+  return fwd_on(a, ws, kStaticScratchBytes, true);
 }
 
 int sba_bwd(const SbaArgs* a) {
@@ -267,7 +311,7 @@ int sba_bwd(const SbaArgs* a) {
   p.vec_ok = v16 ? 1 : 0;
   // The key-tile list is built for the dK/dV kernel that will run (the fp32 kernels do not use it).
   const int key_tile = a->dtype == SBA_F32 ? kBlockK : sba::dkv_key_tile(p);
-  if ((st = run_sched(a, L, true, true, key_tile, stream)) != SBA_OK) return st;
+  if ((st = run_sched(a, ws, L, true, true, key_tile, stream)) != SBA_OK) return st;
   hipEvent_t* ev = (hipEvent_t*)a->trace_events;
   if (ev && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;
   if (a->dtype == SBA_F32) {

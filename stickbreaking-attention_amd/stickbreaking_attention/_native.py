@@ -54,7 +54,7 @@ class SbaPlan(ctypes.Structure):
                 ("pairs", ctypes.c_int64)]
 
 
-EXPORTS = ("sba_version", "sba_strerror", "sba_workspace_bytes", "sba_plan_host", "sba_fwd", "sba_bwd")
+EXPORTS = ("sba_version", "sba_strerror", "sba_workspace_bytes", "sba_plan_host", "sba_fwd", "sba_fwd_static", "sba_bwd")
 STATUS_OFFSET = 8        # SBA_STATUS_OFFSET: the scheduler's status word inside the workspace
 # Debugging aid for the tests: fill the carry buffer and the workspaces with NaN bit patterns before every launch,
 # so that a kernel reading a slot nobody wrote shows up as NaN instead of passing on whatever the allocator returned.
@@ -81,7 +81,7 @@ def lib():
         handle.sba_workspace_bytes.argtypes = [ctypes.POINTER(SbaArgs)] + [ctypes.POINTER(ctypes.c_size_t)] * 3
         handle.sba_plan_host.restype = ctypes.c_int
         handle.sba_plan_host.argtypes = [ctypes.POINTER(SbaArgs), ctypes.c_void_p, ctypes.POINTER(SbaPlan)]
-        for name in ("sba_fwd", "sba_bwd"):
+        for name in ("sba_fwd", "sba_fwd_static", "sba_bwd"):
             fn = getattr(handle, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.POINTER(SbaArgs)]
