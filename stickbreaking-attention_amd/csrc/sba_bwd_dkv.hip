@@ -12,6 +12,7 @@
 // place of the reference's spin-locked read-modify-write of 16-bit dK/dV tiles
 // (stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:11-53, :450-465).
 #include "sba_device.hpp"
+#include "sba_host.hpp"
 #include "sba_params.hpp"
 
 #include <atomic>
@@ -19,29 +20,12 @@
 
 namespace sba {
 
-// Launch facts that do not change while the process lives, looked up once per device instead of on every call:
-// the compute-unit count, and which kernels have had their dynamic-LDS limit raised on which device.
-static hipError_t device_cus(int* dev_out, int* cus_out) {
-  static std::atomic<int> cached[64];
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  int cus = (dev >= 0 && dev < 64) ? cached[dev].load(std::memory_order_relaxed) : 0;
-  if (cus == 0) {
-    if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
-    if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
-  }
-  *dev_out = dev; *cus_out = cus;
-  return hipSuccess;
-}
-template <typename Kernel>
-static hipError_t raise_lds_limit(Kernel kernel, std::atomic<uint64_t>& done, int dev, size_t lds_bytes) {
-  const uint64_t bit = (dev >= 0 && dev < 64) ? (uint64_t)1 << dev : 0;
-  if (bit && (done.load(std::memory_order_acquire) & bit)) return hipSuccess;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-  if (e == hipSuccess && bit) done.fetch_or(bit, std::memory_order_release);
-  return e;
-}
+#ifndef SBA_DKV_LEAD
+#define SBA_DKV_LEAD 24
+#endif
+#ifndef SBA_DKV_SPAN
+#define SBA_DKV_SPAN 240
+#endif
 
 template <int DH> struct DkvLds {
   static constexpr int kRowStride = lds_stride<DH>();
@@ -575,10 +559,6 @@ template <int DH> struct Dkv4Lds {
   static constexpr int kElems = kScratch + 4 * 32 * lds_stride<32>();
 };
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the vector-memory counter, which
-// would stall on the global loads that are deliberately left in flight across the barrier (staging registers,
-// next tile's operands).  Nothing in this kernel communicates through global memory.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 template <typename T, int DH>
 __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
@@ -691,11 +671,11 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
       auto fused = [&](auto diag_tag, int st, const f32x16& s_cur, const f32x16& dp_cur, f32x16& s_next, f32x16& dp_next,
                        int lim, float drem, float prod_in, float prefix_in, uint32_t (&pk)[8], uint32_t (&dzk)[8]) {
         constexpr bool kDiag = decltype(diag_tag)::value;
-        constexpr int kLead = 24;                              // vector-ALU instructions ahead of the first MFMA
+        constexpr int kLead = SBA_DKV_LEAD;                    // vector-ALU instructions ahead of the first MFMA
         // Vector-ALU instructions per MFMA.  The group solver is greedy: with a budget a little below the block's
         // instruction count it puts the last MFMAs back to back and the rest of the math behind them, so the values
         // were checked in the generated code (both element types, both copies of the unrolled step).
-        constexpr int kGap = (kDiag ? 270 : 240) / (2 * kSteps);
+        constexpr int kGap = (kDiag ? SBA_DKV_SPAN + 30 : SBA_DKV_SPAN) / (2 * kSteps);
         constexpr int kAlu = 0x402;                            // scheduling-group mask: vector ALU incl. transcendentals
         const T* q_lds = lds + Lds::kQ + st * 2 * Lds::kQdoTile;
         const T* do_lds = q_lds + Lds::kQdoTile;
@@ -777,9 +757,13 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
       lds_barrier();                                         // the barrier of the last step
     }  // tile walk (producers)
   } else {
+    // Consumer wave (out, cp) owns, for ALL 128 keys of the tile, the columns 32*kCT*cp .. +32*kCT-1 of ONE of the two
+    // outputs: dV (out = 0: P^T dO) or dK (out = 1: dZ^T Q).  Per 16 rows that is 4 weight operands + kCT row operands
+    // for 4*kCT MFMAs: the LDS transpose reads, which bound this kernel, are a quarter fewer than with a wave that
+    // holds 64 keys of both outputs.
     constexpr int kCT = DH / 64;                             // 32-column blocks per consumer wave
-    const int mp = wave >> 1, cp = wave & 1;                 // keys 64*mp .. +63, columns 32*kCT*cp .. +32*kCT-1
-    f32x16 dkacc[2][kCT], dvacc[2][kCT];
+    const int out = wave >> 1, cp = wave & 1;
+    f32x16 acc[4][kCT];
     // Two sets of staging registers, used alternately: a step's rows are requested two steps before they are
     // written to LDS (a step is shorter than a global load).
     TileCopy<T, DH, kRows, true> cq[2], cdo[2];
@@ -797,20 +781,21 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
     };
     if (w < n_tiles) stage_first(next_tile);
     // The results of a tile are stored during the first step of the NEXT tile, when the consumers have nothing to
-    // contract yet (and after the last tile): acc[m][n][r] is key origin + 64*mp + 32*m + 8*(r/4) + 4*half + r%4,
+    // contract yet (and after the last tile): acc[m][n][r] is key origin + 32*m + 8*(r/4) + 4*half + r%4,
     // column 32*(kCT*cp + n) + col.
     bool pending = false;
     Tile done_tile = next_tile;
     auto store_results = [&](const Tile& tl) {
-      const int tl_len = tl.seq_len, tl_j0 = tl.origin + 64 * mp;
+      const int tl_len = tl.seq_len, tl_j0 = tl.origin;
       const int64_t tl_tok0 = tl.seq_start;
-      T* dkb = (T*)p.dk.ptr + tl.seq_id * p.dk.sb + head * p.dk.sh + tl_tok0 * p.dk.st;
-      T* dvb = (T*)p.dv.ptr + tl.seq_id * p.dv.sb + head * p.dv.sh + tl_tok0 * p.dv.st;
-      if (p.add_rem) {
+      T* outb = out ? (T*)p.dk.ptr + tl.seq_id * p.dk.sb + head * p.dk.sh + tl_tok0 * p.dk.st
+                    : (T*)p.dv.ptr + tl.seq_id * p.dv.sb + head * p.dv.sh + tl_tok0 * p.dv.st;
+      const int64_t out_st = out ? p.dk.st : p.dv.st;
+      if (p.add_rem && out == 0) {
         // the remainder term o += rem * v contributes rem_j * d_o_j to dv_j
         const T* dob = (const T*)p.d_o.ptr + tl.seq_id * p.d_o.sb + head * p.d_o.sh + tl_tok0 * p.d_o.st;
 #pragma unroll
-        for (int m = 0; m < 2; m++)
+        for (int m = 0; m < 4; m++)
 #pragma unroll
           for (int r = 0; r < 16; r++) {
             const int key = tl_j0 + 32 * m + 8 * (r >> 2) + 4 * half + (r & 3);
@@ -818,19 +803,18 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
               const float rem = fast_exp2(p.row_stat[tl.seq_id * p.stat_sb + head * p.stat_sh + tl_tok0 + key]);
 #pragma unroll
               for (int n = 0; n < kCT; n++)
-                dvacc[m][n][r] += rem * (float)dob[(int64_t)key * p.d_o.st + 32 * (kCT * cp + n) + col];
+                acc[m][n][r] += rem * (float)dob[(int64_t)key * p.d_o.st + 32 * (kCT * cp + n) + col];
             }
           }
       }
-      const RowSink<T> dk_sink = make_row_sink<T>(dkb, p.dk.st, tl_len, DH), dv_sink = make_row_sink<T>(dvb, p.dv.st, tl_len, DH);
+      const RowSink<T> sink = make_row_sink<T>(outb, out_st, tl_len, DH);
+      const float scale = out ? p.logit_scale : 1.f;
       T* scratch = lds + Lds::kScratch + wave * (32 * lds_stride<32>());
 #pragma unroll
-      for (int m = 0; m < 2; m++)
+      for (int m = 0; m < 4; m++)
 #pragma unroll
-        for (int n = 0; n < kCT; n++) {
-          store_acc_tile_wide<T>(dk_sink, dkacc[m][n], p.logit_scale, tl_j0 + 32 * m, 32 * (kCT * cp + n), half, col, lane, scratch);
-          store_acc_tile_wide<T>(dv_sink, dvacc[m][n], 1.f, tl_j0 + 32 * m, 32 * (kCT * cp + n), half, col, lane, scratch);
-        }
+        for (int n = 0; n < kCT; n++)
+          store_acc_tile_wide<T>(sink, acc[m][n], scale, tl_j0 + 32 * m, 32 * (kCT * cp + n), half, col, lane, scratch);
     };
     for (int slot = w; slot < n_tiles;) {
       const Tile tile = next_tile;
@@ -864,11 +848,11 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
       if (pending) store_results(done_tile);
       stage_rows(2);
 #pragma unroll
-      for (int m = 0; m < 2; m++)
+      for (int m = 0; m < 4; m++)
 #pragma unroll
         for (int n = 0; n < kCT; n++)
 #pragma unroll
-          for (int r = 0; r < 16; r++) { dkacc[m][n][r] = 0.f; dvacc[m][n][r] = 0.f; }
+          for (int r = 0; r < 16; r++) acc[m][n][r] = 0.f;
       lds_barrier();
       for (int t = 1; t <= n_steps; ++t) {
         stage_rows(t + 2);
@@ -877,28 +861,21 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
         const T* do_lds = q_lds + Lds::kQdoTile;
         const T* p_lds = lds + Lds::kP + (u & 1) * 2 * Lds::kPTile;
         const T* dz_lds = p_lds + Lds::kPTile;
-        // dV[key][d] += sum_i P[i][key] dO[i][d];  dK[key][d] += sum_i dZ[i][key] Q[i][d]   (i over the 32 rows)
+        // dV[key][d] += sum_i P[i][key] dO[i][d]  or  dK[key][d] += sum_i dZ[i][key] Q[i][d]   (i over the 32 rows)
+        const T* w_lds = out ? dz_lds : p_lds;               // weights: [row][key]
+        const T* r_lds = out ? q_lds : do_lds;               // rows:    [row][column]
 #pragma unroll
         for (int c = 0; c < kRows / 16; c++) {
           const int row0 = 16 * c + 8 * half;
-          vec8 ap[2], az[2], bd[kCT], bq[kCT];
+          vec8 aw[4], br[kCT];
 #pragma unroll
-          for (int m = 0; m < 2; m++) {
-            ap[m] = lds_col8<T>(p_lds, kPStride, row0, 64 * mp + 32 * m, lane);
-            az[m] = lds_col8<T>(dz_lds, kPStride, row0, 64 * mp + 32 * m, lane);
-          }
+          for (int m = 0; m < 4; m++) aw[m] = lds_col8<T>(w_lds, kPStride, row0, 32 * m, lane);
 #pragma unroll
-          for (int n = 0; n < kCT; n++) {
-            bd[n] = lds_col8<T>(do_lds, kRowStride, row0, 32 * (kCT * cp + n), lane);
-            bq[n] = lds_col8<T>(q_lds, kRowStride, row0, 32 * (kCT * cp + n), lane);
-          }
+          for (int n = 0; n < kCT; n++) br[n] = lds_col8<T>(r_lds, kRowStride, row0, 32 * (kCT * cp + n), lane);
 #pragma unroll
-          for (int m = 0; m < 2; m++)
+          for (int m = 0; m < 4; m++)
 #pragma unroll
-            for (int n = 0; n < kCT; n++) {
-              dvacc[m][n] = Elem<T>::mfma(ap[m], bd[n], dvacc[m][n]);
-              dkacc[m][n] = Elem<T>::mfma(az[m], bq[n], dkacc[m][n]);
-            }
+            for (int n = 0; n < kCT; n++) acc[m][n] = Elem<T>::mfma(aw[m], br[n], acc[m][n]);
         }
         lds_barrier();
       }

@@ -358,6 +358,11 @@ __device__ __forceinline__ void zero_rows(const TensorRef& t, int head, int64_t 
   for (int64_t idx = threadIdx.x; idx < n; idx += blockDim.x) b[(r0 + idx / d) * t.st + idx % d] = (T)0;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the vector-memory counter, which
+// would stall on global loads that are deliberately left in flight across the barrier (staging registers, the next
+// tile's operands).  For kernels in which nothing is communicated through global memory.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Map the linear workgroup id to (head, tile slot) so that the workgroups of one head land on one XCD
 // (workgroups are dealt round-robin to the 8 XCDs, each with a private L2): K/V of a head are then
 // re-read from that XCD's L2 rather than from HBM.

@@ -17,6 +17,14 @@
 
 namespace sba {
 
+#ifndef SBA_FWD_KAHEAD
+#define SBA_FWD_KAHEAD 1
+#endif
+#ifndef SBA_FWD_VHOIST
+#define SBA_FWD_VHOIST 0
+#endif
+constexpr bool kKAhead = SBA_FWD_KAHEAD, kVHoist = SBA_FWD_VHOIST;
+
 template <typename T, int DH, bool kFast, int KT, int kMinWaves>
 __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
   constexpr int NT = KT / 32;         // MFMA row tiles per key tile: a lane owns N = 16*NT consecutive keys
@@ -109,10 +117,25 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) s[mt][r] = 0.f;
       const int krow = NT == 2 ? mfma_row_to_key(mt, col) : mfma_row_to_key32(col);
+      if (NT == 1 && kFast && kKAhead) {
+        // The K operands are requested four ahead of the MFMA that uses them: requested two at a time (what the
+        // register allocator otherwise settles for) the wave pays the LDS latency four times per step.
+        vec8 a[kSteps];
 #pragma unroll
-      for (int kk = 0; kk < kSteps; kk++) {
-        vec8 a = lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half);
-        s[mt] = Elem<T>::mfma(a, qf[kk], s[mt]);
+        for (int kk = 0; kk < 4; kk++) a[kk] = lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < kSteps; kk++) {
+          s[mt] = Elem<T>::mfma(a[kk], qf[kk], s[mt]);
+          if (kk + 4 < kSteps) a[kk + 4] = lds_row8<T>(k_lds, kRowStride, krow, 16 * (kk + 4) + 8 * half);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+#pragma unroll
+        for (int kk = 0; kk < kSteps; kk++) {
+          vec8 a = lds_row8<T>(k_lds, kRowStride, krow, 16 * kk + 8 * half);
+          s[mt] = Elem<T>::mfma(a, qf[kk], s[mt]);
+        }
       }
     }
 
@@ -121,6 +144,13 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
     // (the weight of key R up to the product carried into the tile).  The difference form needs neither sigma
     // nor a clamp: e = inf gives a factor 0 and the whole remaining stick as weight; its absolute error is one
     // ulp of the running product.  Hidden keys (diagonal tiles only) get e = 0: factor 1, weight 0.
+    // The V operands of the first 16 keys are requested before the element-wise math, which covers their latency.
+    vec8 vfirst[kDTiles];
+    if (NT == 1 && kFast && kVHoist) {
+#pragma unroll
+      for (int dt = 0; dt < kDTiles; dt++) vfirst[dt] = lds_col8<T>(v_lds, kRowStride, N * half, 32 * dt, lane);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     float t[N];
     float run = 1.f;
     if (diagonal) {
@@ -156,7 +186,7 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
       vec8 a = as_vec8<T>(av);
 #pragma unroll
       for (int dt = 0; dt < kDTiles; dt++) {
-        vec8 b = lds_col8<T>(v_lds, kRowStride, N * half + 8 * c, 32 * dt, lane);
+        vec8 b = (NT == 1 && kFast && kVHoist && c == 0) ? vfirst[dt] : lds_col8<T>(v_lds, kRowStride, N * half + 8 * c, 32 * dt, lane);
         oacc[dt] = Elem<T>::mfma(a, b, oacc[dt]);
       }
     }
