@@ -28,11 +28,20 @@ sys.path.insert(0, os.path.join(ROOT, "stickbreaking-attention_amd"))
 
 MFMA_BF16_PEAK = 2.5e15          # MI355X dense bf16 MFMA peak, FLOP/s
 
-# HBM bytes per launch (fetch + write) of each kernel on workload c3, from `rocprofv3 --pmc FETCH_SIZE` and
-# `--pmc WRITE_SIZE` runs of `bench.py --traffic-probe`, each scaled by what the same counter read for the probe's
-# 1 GiB device-to-device copy.  Hardware counters cannot be read from inside this script, so the figures are carried
-# here; they are reported only for the workload they were measured on.
-MEASURED_TRAFFIC_BYTES = {"c3": {"fwd_kernel": 2.059e9, "bwd_dq_kernel": 1.950e9, "bwd_dkv_kernel": 2.616e9}}
+# HBM bytes per launch (fetch + write) of each kernel cannot be read from inside this script (hardware counters need
+# rocprofv3): they are measured by the two `rocprofv3 --pmc` runs whose summary is profiles/c3_varlen_hbm_traffic_pmc.txt
+# and kept, with the commit they were measured at, in the JSON file beside that summary.  `roofline.traffic` reports
+# the figure for the dominant kernel of the workload it was measured on, null otherwise.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def measured_traffic(workload, kernel):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+        return rec["bytes_per_launch"][workload][kernel]
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 # ----------------------------------------------------------------------------------------------
@@ -150,14 +159,24 @@ def time_kernels(inp, native, iters):
 
 
 def cpu_baseline(sample_len=4096, budget_s=15.0):
-    """The CPU restatement (dense fp32 forward + autograd backward) timed on (head, sequence) slices of the bench
-    workload's shape, one after another until about `budget_s` seconds of CPU work have been spent."""
+    """The CPU restatement (dense fp32 forward + autograd backward, the same operations as sb_ref.py including its
+    L x L contraction) timed on the host: configuration C1 in full (fp32, 4 heads, head_dim 64, lengths [128, 256, 64]),
+    then (head, sequence) slices of the bench workload's shape, one after another until about `budget_s` seconds of
+    CPU work have been spent.  `value` is the rate on the slices."""
     sys.path.insert(0, ROOT)
     from oracle import sb_oracle as orc
 
+    threads = torch.get_num_threads()
+    c1 = make_inputs("c1", "cpu")
+    orc.dense_backward_autograd(c1["q"], c1["k"], c1["v"], c1["cu"], c1["do"], c1["drem"])          # warm-up
+    reps, t0 = 5, time.perf_counter()
+    for _ in range(reps):
+        orc.dense_backward_autograd(c1["q"], c1["k"], c1["v"], c1["cu"], c1["do"], c1["drem"])
+    c1_ms = (time.perf_counter() - t0) * 1e3 / reps
+    c1_tflops = 14 * c1["D"] * visible_pairs(c1["lengths"], c1["H"]) / (c1_ms * 1e-3) / 1e12
+
     D = 128
     g = torch.Generator().manual_seed(0)
-    threads = torch.get_num_threads()
     slices, spent = 0, 0.0
     while spent < budget_s:
         q, k, v, do = (torch.randn(1, sample_len, D, generator=g) for _ in range(4))
@@ -169,7 +188,8 @@ def cpu_baseline(sample_len=4096, budget_s=15.0):
     flops = 14 * D * visible_pairs([sample_len], 1) * slices
     return {"value": flops / spent / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "sample": f"fwd+bwd of {slices} (head, sequence) slices, L={sample_len}, D=128, fp32 dense restatement of "
-                      f"sb_ref.py via autograd, {spent:.1f} s, os.cpu_count()={os.cpu_count()}"}
+                      f"sb_ref.py via autograd, {spent:.1f} s, os.cpu_count()={os.cpu_count()}; configuration C1 in full "
+                      f"(fp32, H=4, D=64, lengths [128, 256, 64], fwd+bwd): {c1_ms:.2f} ms = {c1_tflops:.4f} TFLOP/s"}
 
 
 def main():
@@ -268,7 +288,7 @@ def main():
         "kernels_ms": {n: round(kernels[n][0], 4) for n in kernels},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": MFMA_BF16_PEAK / 1e12, "unit": "TFLOP/s",
                      "frac": achieved * 1e12 / MFMA_BF16_PEAK,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dom)},
+                     "traffic": measured_traffic(args.workload, dom)},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()

@@ -21,6 +21,7 @@ What it restates (citations are into the reference repository):
   form dz_ij = g_ij - sigmoid(z_ij) * sum_{j'<=j} g_ij', g_ij = A_ij (do_i.v_j - drem_i), which is
   what stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:438-452 evaluates tile by tile.
 
+* ``stream_rowblocked``        -- the streaming form a block of query rows at a time (for 64K-token sequences).
 * ``rounding_floor``           -- the streaming form evaluated in float64 with exactly two kinds of rounding
   put back: the weights P and the logit gradient dZ are rounded to the 16-bit input type before they are
   contracted (the reference rounds at the same points: sb_varlen_fwd.py:193 ``p.to(v.dtype)``,
@@ -146,6 +147,51 @@ def stream_backward(q, k, v, do, drem, scale=None, attend_current=False):
     dk = torch.matmul(dz.transpose(-1, -2), q) * scale
     dv = torch.matmul(att.transpose(-1, -2), do)
     return dq, dk, dv
+
+
+def stream_rowblocked(q, k, v, do=None, drem=None, scale=None, attend_current=False, block=2048, dtype=torch.float32,
+                      rows: Optional[Tuple[int, int]] = None):
+    """``stream_forward`` / ``stream_backward`` of ONE (L, D) problem evaluated a block of query rows at a time, so that
+    a 64K-token sequence needs (block x L) matrices instead of (L x L): rows are independent in o, rem and dq, and
+    dk, dv are sums over row blocks.  Same formulas, same results to rounding (pinned against the unblocked form).
+    ``rows = (r0, r1)`` evaluates only those query rows: o, rem, dq are then complete for them (and zero elsewhere),
+    dk and dv hold only those rows' contributions."""
+    if scale is None:
+        scale = 1.0 / math.sqrt(q.shape[-1])
+    L, D = q.shape
+    q, k, v = (t.to(dtype) for t in (q, k, v))
+    o = torch.zeros(L, D, dtype=dtype)
+    rem = torch.zeros(L, dtype=dtype)
+    grads = None
+    if do is not None:
+        do = do.to(dtype)
+        drem = torch.zeros(L, dtype=dtype) if drem is None else drem.to(dtype)
+        grads = [torch.zeros(L, D, dtype=dtype) for _ in range(3)]
+    first, last = (0, L) if rows is None else rows
+    for r0 in range(first, last, block):
+        r1 = min(r0 + block, last)
+        nk = min(r1 if attend_current else r1 - 1, L)          # keys any row of the block can see
+        if nk <= 0:
+            rem[r0:r1] = 1
+            continue
+        i = torch.arange(r0, r1)[:, None]
+        j = torch.arange(nk)[None, :]
+        vis = (j <= i) if attend_current else (j < i)
+        z = torch.matmul(q[r0:r1], k[:nk].T) * scale
+        log_skip = torch.where(vis, -F.softplus(z), torch.zeros_like(z))
+        suffix = log_skip.flip(-1).cumsum(-1).flip(-1) - log_skip
+        att = torch.where(vis, (F.logsigmoid(z) + suffix).exp(), torch.zeros_like(z))
+        o[r0:r1] = torch.matmul(att, v[:nk])
+        rem[r0:r1] = log_skip.sum(-1).exp()
+        if grads is not None:
+            g = att * (torch.matmul(do[r0:r1], v[:nk].T) - drem[r0:r1, None])
+            dz = torch.where(vis, g - torch.sigmoid(z) * g.cumsum(-1), torch.zeros_like(z))
+            grads[0][r0:r1] = torch.matmul(dz, k[:nk]) * scale
+            grads[1][:nk] += torch.matmul(dz.T, q[r0:r1]) * scale
+            grads[2][:nk] += torch.matmul(att.T, do[r0:r1])
+    if grads is None:
+        return o, rem
+    return (o, rem, *grads)
 
 
 def varlen_stream(q, k, v, cu_seqlens, scale=None, zero_start=False, attend_current=False,

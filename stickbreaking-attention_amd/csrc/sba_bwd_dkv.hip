@@ -20,13 +20,6 @@
 
 namespace sba {
 
-#ifndef SBA_DKV_LEAD
-#define SBA_DKV_LEAD 24
-#endif
-#ifndef SBA_DKV_SPAN
-#define SBA_DKV_SPAN 240
-#endif
-
 template <int DH> struct DkvLds {
   static constexpr int kRowStride = lds_stride<DH>();
   static constexpr int kPStride = lds_stride<kBlockK>();
@@ -671,11 +664,11 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
       auto fused = [&](auto diag_tag, int st, const f32x16& s_cur, const f32x16& dp_cur, f32x16& s_next, f32x16& dp_next,
                        int lim, float drem, float prod_in, float prefix_in, uint32_t (&pk)[8], uint32_t (&dzk)[8]) {
         constexpr bool kDiag = decltype(diag_tag)::value;
-        constexpr int kLead = SBA_DKV_LEAD;                    // vector-ALU instructions ahead of the first MFMA
+        constexpr int kLead = 24;                              // vector-ALU instructions ahead of the first MFMA
         // Vector-ALU instructions per MFMA.  The group solver is greedy: with a budget a little below the block's
         // instruction count it puts the last MFMAs back to back and the rest of the math behind them, so the values
         // were checked in the generated code (both element types, both copies of the unrolled step).
-        constexpr int kGap = (kDiag ? SBA_DKV_SPAN + 30 : SBA_DKV_SPAN) / (2 * kSteps);
+        constexpr int kGap = (kDiag ? 270 : 240) / (2 * kSteps);
         constexpr int kAlu = 0x402;                            // scheduling-group mask: vector ALU incl. transcendentals
         const T* q_lds = lds + Lds::kQ + st * 2 * Lds::kQdoTile;
         const T* do_lds = q_lds + Lds::kQdoTile;

@@ -177,3 +177,31 @@ def test_torch_compile_against_oracle(gpu_device, backend):
     torch.cuda.synchronize()
     for n, a, b in zip(NAMES, (o.detach(), rem.detach(), q.grad, k.grad, v.grad), ref):
         tol_check(n, a, b, torch.bfloat16, f"compiled fixed ({backend})")
+
+
+def test_single_sequence_of_64k_tokens(gpu_device, poisoned):
+    """One 65536-token sequence, one head: the length at which the per-(row, 32-key sub-tile) planes the backward works
+    from (L^2 / 16 bytes per head each) are the largest buffers in play, sized exactly from the host lengths.  o, rem
+    and dq are checked against the row-blocked oracle on the first, a middle and the last 2048 rows (rows are
+    independent in those three); dk and dv, which sum over all rows, against the library's fp32 vector-ALU path on the
+    same values -- a separate implementation pinned by its own oracle tests -- and the forward outputs against it too."""
+    from stickbreaking_attention import _native
+
+    L, D = 65536, 128
+    g = torch.Generator().manual_seed(61)
+    q, k, v, do = (torch.randn(1, L, D, generator=g).bfloat16() for _ in range(4))
+    drem = torch.randn(1, L, generator=g).bfloat16()
+    cu = torch.tensor([L], dtype=torch.int32)
+    plan = _native.plan_host(cu, False, L)
+    assert plan.carry_slots == 256 * 512 * 513 and plan.pairs == L * (L - 1) // 2
+    dev = [t.to(gpu_device) for t in (q, k, v, do, drem)]
+    got = run_varlen(*dev[:3], cu, [L], False, False, dev[3], dev[4])          # host cu_seqlens: exact buffer sizes
+    for t in got:
+        assert torch.isfinite(t.float()).all()
+    for r0 in (0, 31744, L - 2048):
+        ref = orc.stream_rowblocked(q[0], k[0], v[0], do[0], drem[0], rows=(r0, r0 + 2048))
+        for n, a, b in zip(NAMES[:3], got[:3], ref[:3]):
+            tol_check(n, a[0, r0:r0 + 2048], b[r0:r0 + 2048], torch.bfloat16, f"64k rows {r0}..{r0 + 2047}")
+    f32 = run_varlen(*(t.float() for t in dev[:3]), cu, [L], False, False, dev[3].float(), dev[4].float())
+    for n, a, b in zip(NAMES, got, f32):
+        tol_check(n, a, b.double().cpu(), torch.bfloat16, "64k vs fp32 path")

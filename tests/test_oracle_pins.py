@@ -356,3 +356,26 @@ def test_rounding_floor_of_saturating_logits_sits_at_the_parity_bound():
         worst = max(worst, excess)
     assert -6e-3 < worst < 6e-3  # at the bound, on one side or the other ...
     assert max((a - b).abs().max().item() for a, b in zip(floor[2:4], exact[2:4])) > 2e-2      # ... and well above 2e-2 absolute
+
+
+@pytest.mark.parametrize("attend_current", [False, True])
+def test_rowblocked_stream_matches_unblocked(attend_current):
+    """`stream_rowblocked` (the checker of the 64K-token GPU test) against the unblocked streaming form, which the tests
+    above pin: block sizes that do and do not divide the length, a block larger than the sequence, length 1."""
+    torch.manual_seed(31)
+    for L, block in ((97, 32), (64, 64), (50, 512), (1, 4), (130, 7)):
+        D = 8
+        q, k, v, do = (torch.randn(L, D, dtype=torch.float64) for _ in range(4))
+        drem = torch.randn(L, dtype=torch.float64)
+        o, rem = orc.stream_forward(q, k, v, 0.3, attend_current)
+        grads = orc.stream_backward(q, k, v, do, drem, 0.3, attend_current)
+        got = orc.stream_rowblocked(q, k, v, do, drem, 0.3, attend_current, block=block, dtype=torch.float64)
+        for a, b in zip(got, (o, rem, *grads)):
+            torch.testing.assert_close(a, b, atol=1e-12, rtol=0)
+        fwd_only = orc.stream_rowblocked(q, k, v, scale=0.3, attend_current=attend_current, block=block, dtype=torch.float64)
+        assert torch.equal(fwd_only[0], got[0]) and torch.equal(fwd_only[1], got[1])
+        if L > 40:          # a window of rows: o, rem, dq complete inside it, untouched outside
+            part = orc.stream_rowblocked(q, k, v, do, drem, 0.3, attend_current, block=block, dtype=torch.float64, rows=(20, 41))
+            for a, b in zip(part[:3], (o, rem, grads[0])):
+                torch.testing.assert_close(a[20:41], b[20:41], atol=1e-12, rtol=0)
+                assert (a[:20] == 0).all() and (a[41:] == 0).all()
