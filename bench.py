@@ -127,8 +127,9 @@ class KernelTimer:
         return ms.value
 
 
-def time_kernels(inp, native, iters):
-    """Average duration of the forward, dQ and dK/dV kernels through the C ABI (scheduler kernel excluded)."""
+def time_kernels(inp, native, iters, save_carry=True):
+    """Average duration of the forward, dQ and dK/dV kernels through the C ABI (scheduler kernel excluded; without
+    saved products the kernel that rebuilds them is timed with the dQ kernel)."""
     timer = KernelTimer(native)
     q, k, v = inp["q"], inp["k"], inp["v"]
     lead0 = inp["zero_start"]
@@ -146,7 +147,7 @@ def time_kernels(inp, native, iters):
     for it in range(iters + 2):
         fwd_ev, bwd_ev = timer.new_set(2), timer.new_set(3)
         native.TRACE_EVENTS = fwd_ev
-        o, rem, row_stat, carry = native.forward(q, k, v, cu, lead0, maxlen, scale, False, want_carry=True)
+        o, rem, row_stat, carry = native.forward(q, k, v, cu, lead0, maxlen, scale, False, want_carry=save_carry)
         native.TRACE_EVENTS = bwd_ev
         native.backward(do, drem, q, k, v, carry, cu, lead0, maxlen, scale, False)
         native.TRACE_EVENTS = None
@@ -199,6 +200,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-saved-carry", action="store_true",
+                    help="keep only q, k, v between the passes (save_carry=False): the backward rebuilds the forward's products")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch one plain 1 GiB device copy, the known-size reference for HBM traffic counters")
     args = ap.parse_args()
@@ -216,15 +219,16 @@ def main():
     H, D, T, lengths = inp["H"], inp["D"], inp["T"], inp["lengths"]
     pairs = visible_pairs(lengths, H)
     q, k, v = (inp[n].requires_grad_() for n in ("q", "k", "v"))
+    save_carry = not args.no_saved_carry
 
     def step():
         if inp["fixed"]:
             B, L = len(lengths), lengths[0]
             q4, k4, v4 = (t.view(H, B, L, D).transpose(0, 1) for t in (q, k, v))
-            o, rem = sb_attn(q4, k4, v4)
+            o, rem = sb_attn(q4, k4, v4, save_carry=save_carry)
             torch.autograd.backward([o, rem], [inp["do"].view(H, B, L, D).transpose(0, 1), inp["drem"].view(H, B, L).transpose(0, 1)])
         else:
-            o, rem = sb_attn_varlen(q, k, v, inp["cu"], max(lengths), zero_start=inp["zero_start"])
+            o, rem = sb_attn_varlen(q, k, v, inp["cu"], max(lengths), zero_start=inp["zero_start"], save_carry=save_carry)
             torch.autograd.backward([o, rem], [inp["do"], inp["drem"]])
         q.grad = k.grad = v.grad = None
 
@@ -261,7 +265,7 @@ def main():
     torch.cuda.synchronize()
     ms_fwd = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    k_fwd, k_dq, k_dkv = time_kernels(inp, _native, max(5, min(args.steps, 20)))
+    k_fwd, k_dq, k_dkv = time_kernels(inp, _native, max(5, min(args.steps, 20)), save_carry)
     # Algorithmic FLOPs per launch: forward QK^T + PV = 4 D pairs; backward 10 D pairs, of which the dQ kernel is
     # credited with the recompute (QK^T, dO V^T) and dQ = 6 D pairs and the dK/dV kernel with dK, dV = 4 D pairs
     # (its own recompute of QK^T and dO V^T is not algorithmic work).
@@ -280,7 +284,8 @@ def main():
         "dtype": str(inp["dtype"]).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32"),
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: sb_attn{'_varlen' if not inp['fixed'] else ''} fwd+bwd, H={H}, D={D}, "
-                               f"T={T}, {len(lengths)} sequences (max {max(lengths)}), pairs={pairs}"},
+                               f"T={T}, {len(lengths)} sequences (max {max(lengths)}), pairs={pairs}"
+                               + ("" if save_carry else ", products rebuilt in the backward")},
         "frac_bf16_mfma_peak": flops_step / (ms_step * 1e-3) / MFMA_BF16_PEAK,
         "tokens_per_s": T / (ms_step * 1e-3),
         "fwd": {"ms": ms_fwd, "tflops": 4 * D * pairs / (ms_fwd * 1e-3) / 1e12, "tokens_per_s": T / (ms_fwd * 1e-3),

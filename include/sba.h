@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 3
+#define SBA_VERSION 4
 
 /* Scheduler status word: int32 at this byte offset of the workspace, valid after the stream has run. */
 #define SBA_STATUS_OFFSET 8
@@ -60,7 +60,7 @@ typedef enum SbaStatus {
   SBA_ERR_STRIDE = -4,      /* a negative stride (any non-negative head/token/batch stride is accepted; strides and
                                base pointers that are multiples of 16 bytes select the fast kernels) */
   SBA_ERR_ALIGN = -5,       /* a tensor base pointer is not aligned to its element size */
-  SBA_ERR_SHAPE = -6,       /* non-positive sizes, total_tokens > 2^30, or a reserved field that is not 0 */
+  SBA_ERR_SHAPE = -6,       /* non-positive sizes, total_tokens > 2^30, a negative carry_slots or a flag outside {0, 1} */
   SBA_ERR_WORKSPACE = -7,   /* workspace missing, not 256-byte aligned, or smaller than sba_workspace_bytes reports */
   SBA_ERR_LAUNCH = -8,      /* the HIP runtime rejected a launch (hipGetLastError) */
   SBA_ERR_TOO_LARGE = -9    /* sba_fwd_static: the tile schedule does not fit the library's static scratch */
@@ -120,7 +120,12 @@ typedef struct SbaArgs {
                                   The backward then takes d_o as the gradient of that sum and d_rem as the
                                   gradient that reaches rem directly, needs row_stat (as the forward wrote it) as an
                                   input, and returns dv including rem * d_o. */
-  int32_t reserved0;           /* must be 0 */
+  int32_t recompute_carry;     /* 0 or 1.  1: the backward does not take `carry` from the forward (which may then be run
+                                  with carry = NULL) but rebuilds it in its own workspace from q and k, with the forward
+                                  kernel stripped of everything else: the state kept between the passes is then O(tokens)
+                                  as in the reference (q, k, v and, with add_remainder, row_stat), at the price of one more
+                                  kernel in the backward.  Must be the same in sba_workspace_bytes and sba_bwd.  16-bit
+                                  dtypes only. */
   int64_t carry_slots;         /* fp32 slots of `carry` (and of the backward's prefix plane) per head.  0: sized from
                                   the bound total_tokens * max_seqlen / 64 (packed mode), which is several times the
                                   need of a ragged batch; a caller that knows the lengths on the host passes

@@ -9,6 +9,7 @@
 namespace sba {
 hipError_t launch_sched(const SchedParams& p, hipStream_t stream);
 hipError_t launch_fwd(const FwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
+hipError_t launch_fwd_carry_only(const FwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
 hipError_t launch_bwd_dq(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
 hipError_t launch_bwd_dkv(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
 int dkv_key_tile(const BwdParams& p);
@@ -26,7 +27,7 @@ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 struct Layout {
   int64_t max_q_tiles, max_k_tiles, carry_slots_per_head;
-  size_t off_counts, off_q_tiles, off_k_tiles, off_carry_base, off_prefix, off_drem, off_queue;
+  size_t off_counts, off_q_tiles, off_k_tiles, off_carry_base, off_prefix, off_drem, off_queue, off_carry;
   size_t fwd_bytes, bwd_bytes, carry_bytes;
 };
 
@@ -35,7 +36,8 @@ int plan(const SbaArgs* a, Layout* out) {
   if (a->head_dim < 1 || a->head_dim > 128) return SBA_ERR_HEAD_DIM;
   if (a->dtype != SBA_BF16 && a->dtype != SBA_F16 && a->dtype != SBA_F32) return SBA_ERR_DTYPE;
   if (a->total_tokens > (int64_t)1 << 30) return SBA_ERR_SHAPE;
-  if (a->reserved0 != 0 || a->carry_slots < 0) return SBA_ERR_SHAPE;
+  if ((a->recompute_carry != 0 && a->recompute_carry != 1) || a->carry_slots < 0) return SBA_ERR_SHAPE;
+  if (a->recompute_carry && a->dtype == SBA_F32) return SBA_ERR_DTYPE;      // the fp32 path always keeps its products
   Layout L{};
   const int64_t T = a->total_tokens, B = a->num_seqs;
   const bool fixed = a->cu_seqlens == nullptr;
@@ -63,6 +65,8 @@ int plan(const SbaArgs* a, Layout* out) {
   // d_rem + d_o . v per row (fp32), used when the remainder term is fused
   L.off_drem = off;        off = align_up(off + (size_t)a->num_heads * (size_t)T * (fixed ? (size_t)B : 1) * sizeof(float), 256);
   L.off_queue = off;       off = align_up(off + (size_t)a->num_heads * sizeof(int32_t), 256);      // per-head tile cursors
+  // the forward's products, rebuilt inside the backward when the caller did not keep them
+  L.off_carry = off;       if (a->recompute_carry) off += L.carry_bytes;
   L.bwd_bytes = off;
   *out = L;
   return SBA_OK;
@@ -271,7 +275,7 @@ int sba_bwd(const SbaArgs* a) {
       (st = check_tensor(a->dq, true, fixed)) || (st = check_tensor(a->dk, true, fixed)) ||
       (st = check_tensor(a->dv, true, fixed)))
     return st;
-  if (!a->carry) return SBA_ERR_NULL;
+  if (!a->carry && !a->recompute_carry) return SBA_ERR_NULL;
   if (a->add_remainder && !a->row_stat) return SBA_ERR_NULL;
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
     if (t->ptr && ((uintptr_t)t->ptr % es)) return SBA_ERR_ALIGN;
@@ -288,7 +292,7 @@ int sba_bwd(const SbaArgs* a) {
   p.k_tiles = (const sba::Tile*)(ws + L.off_k_tiles);
   p.counts = (const int32_t*)(ws + L.off_counts);
   p.carry_base = (const int64_t*)(ws + L.off_carry_base);
-  p.carry = a->carry;
+  p.carry = a->recompute_carry ? (const float*)(ws + L.off_carry) : a->carry;
   p.prefix = (float*)(ws + L.off_prefix);
   p.carry_head_stride = L.carry_slots_per_head;
   p.num_heads = a->num_heads;
@@ -318,6 +322,27 @@ int sba_bwd(const SbaArgs* a) {
     if (sba::launch_bwd_f32(p, fixed ? a->num_seqs : 1, a->total_tokens, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
     if (ev && (hipEventRecord(ev[1], stream) != hipSuccess || hipEventRecord(ev[2], stream) != hipSuccess)) return SBA_ERR_LAUNCH;
     return SBA_OK;
+  }
+  if (a->recompute_carry) {
+    // O(L) state between the passes: the products the forward would have recorded are rebuilt from q and k by the
+    // forward kernel stripped of everything else (timed with the dQ kernel by trace_events).
+    sba::FwdParams f{};
+    f.q = p.q; f.k = p.k; f.v = p.v; f.o = p.q;
+    f.carry = (float*)(ws + L.off_carry);
+    f.carry_base = p.carry_base;
+    f.carry_head_stride = L.carry_slots_per_head;
+    f.tiles = p.q_tiles;
+    f.counts = p.counts;
+    f.num_heads = a->num_heads;
+    f.head_dim = a->head_dim;
+    f.scale_log2 = p.scale_log2;
+    f.attend_current = p.attend_current;
+    f.max_tiles = (int32_t)L.max_q_tiles;
+    f.total_tokens = a->total_tokens;
+    bool fv16 = (a->head_dim % (16 / (int)es)) == 0;
+    for (const SbaTensor* t : {&a->q, &a->k}) fv16 = fv16 && vec16(*t, es, fixed, max_rows);
+    f.vec_ok = fv16 ? 1 : 0;
+    if (sba::launch_fwd_carry_only(f, a->dtype == SBA_F16, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
   }
   if (sba::launch_bwd_dq(p, a->dtype == SBA_F16, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
   if (ev && hipEventRecord(ev[1], stream) != hipSuccess) return SBA_ERR_LAUNCH;

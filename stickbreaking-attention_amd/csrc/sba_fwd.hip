@@ -17,15 +17,9 @@
 
 namespace sba {
 
-#ifndef SBA_FWD_KAHEAD
-#define SBA_FWD_KAHEAD 1
-#endif
-#ifndef SBA_FWD_VHOIST
-#define SBA_FWD_VHOIST 0
-#endif
-constexpr bool kKAhead = SBA_FWD_KAHEAD, kVHoist = SBA_FWD_VHOIST;
-
-template <typename T, int DH, bool kFast, int KT, int kMinWaves>
+// kCarryOnly: only the products of (1 - sigma) above every sub-tile are rebuilt (into `carry`), for a backward whose
+// forward did not keep them: no V, no P V, no outputs.
+template <typename T, int DH, bool kFast, int KT, int kMinWaves, bool kCarryOnly = false>
 __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
   constexpr int NT = KT / 32;         // MFMA row tiles per key tile: a lane owns N = 16*NT consecutive keys
   constexpr int N = 16 * NT;
@@ -40,7 +34,7 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
   xcd_head_tile(blockIdx.x, p.num_heads, &head, &slot);
   if (slot >= p.counts[kCountQ]) {
     int64_t r0, r1;
-    if (uncovered_rows(p.counts, slot, p.total_tokens, 0, kBlockQ, &r0, &r1)) {      // rows of no sequence: o = rem = 0
+    if (!kCarryOnly && uncovered_rows(p.counts, slot, p.total_tokens, 0, kBlockQ, &r0, &r1)) {      // rows of no sequence: o = rem = 0
       zero_rows<T>(p.o, head, r0, r1, p.head_dim);
       for (int64_t r = r0 + threadIdx.x; r < r1; r += kThreads) {
         ((T*)p.rem.ptr)[head * p.rem.sh + r * p.rem.st] = (T)0;
@@ -82,7 +76,7 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
   TileCopy<T, DH, KT, kFast> ck, cv;
   if (n_kt > 0) {
     ck.load(ksrc, (n_kt - 1) * KT);
-    cv.load(vsrc, (n_kt - 1) * KT);
+    if (!kCarryOnly) cv.load(vsrc, (n_kt - 1) * KT);
   }
   // The recorded products are read per 64-key tile by the backward kernels that sweep 64 keys at a time, whichever
   // forward variant ran: a 32-key sweep that ends on the lower half of such a tile also records the (empty) product
@@ -92,12 +86,12 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
     const int j0 = jt * KT;
     __syncthreads();
     ck.store(k_lds);
-    cv.store(v_lds);
+    if (!kCarryOnly) cv.store(v_lds);
     __syncthreads();
     if (jt > 0) {
       const int jn = j0 - KT;
       ck.load(ksrc, jn);
-      cv.load(vsrc, jn);
+      if (!kCarryOnly) cv.load(vsrc, jn);
     }
     // For the backward: the product over the keys between the upper 32-key sub-tile and the row, for every row
     // of the tile (the lower sub-tile's value follows once this tile's upper half is known).
@@ -117,7 +111,7 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) s[mt][r] = 0.f;
       const int krow = NT == 2 ? mfma_row_to_key(mt, col) : mfma_row_to_key32(col);
-      if (NT == 1 && kFast && kKAhead) {
+      if (NT == 1 && kFast) {
         // The K operands are requested four ahead of the MFMA that uses them: requested two at a time (what the
         // register allocator otherwise settles for) the wave pays the LDS latency four times per step.
         vec8 a[kSteps];
@@ -144,13 +138,6 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
     // (the weight of key R up to the product carried into the tile).  The difference form needs neither sigma
     // nor a clamp: e = inf gives a factor 0 and the whole remaining stick as weight; its absolute error is one
     // ulp of the running product.  Hidden keys (diagonal tiles only) get e = 0: factor 1, weight 0.
-    // The V operands of the first 16 keys are requested before the element-wise math, which covers their latency.
-    vec8 vfirst[kDTiles];
-    if (NT == 1 && kFast && kVHoist) {
-#pragma unroll
-      for (int dt = 0; dt < kDTiles; dt++) vfirst[dt] = lds_col8<T>(v_lds, kRowStride, N * half, 32 * dt, lane);
-      __builtin_amdgcn_sched_barrier(0);
-    }
     float t[N];
     float run = 1.f;
     if (diagonal) {
@@ -176,6 +163,7 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
     const float seed = half ? prod : prod * oth;
     if (NT == 2 && carry && half == 0) carry[carry_offset(u_hi - 1, n_qt) + cslot] = seed;   // product above the lower sub-tile
     prod = (prod * oth) * run;
+    if (kCarryOnly) continue;
 
     // O += P V: A = P from registers (k index <-> key 32*half + 8c + t), B = V gathered down the keys.
 #pragma unroll
@@ -186,12 +174,13 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
       vec8 a = as_vec8<T>(av);
 #pragma unroll
       for (int dt = 0; dt < kDTiles; dt++) {
-        vec8 b = (NT == 1 && kFast && kVHoist && c == 0) ? vfirst[dt] : lds_col8<T>(v_lds, kRowStride, N * half + 8 * c, 32 * dt, lane);
+        vec8 b = lds_col8<T>(v_lds, kRowStride, N * half + 8 * c, 32 * dt, lane);
         oacc[dt] = Elem<T>::mfma(a, b, oacc[dt]);
       }
     }
   }
 
+  if (kCarryOnly) return;
   // Epilogue.  oacc[dt][r]: query row 8*(r/4) + 4*half + r%4 of this wave, column 32*dt + col.
   T* ob = (T*)p.o.ptr + tile.seq_id * p.o.sb + head * p.o.sh + (int64_t)tile.seq_start * p.o.st;
   if (p.add_rem) {
@@ -231,24 +220,30 @@ __global__ __launch_bounds__(kThreads, kMinWaves) void fwd_kernel(FwdParams p) {
   }
 }
 
-template <typename T>
+template <typename T, bool kCarryOnly>
 static hipError_t launch_fwd_t(const FwdParams& p, int max_tiles, hipStream_t stream) {
   const dim3 grid((unsigned)(max_tiles * p.num_heads)), block(kThreads);
   if (p.vec_ok && p.head_dim == 128) {
-    hipLaunchKernelGGL((fwd_kernel<T, 128, true, 32, 3>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<T, 128, true, 32, 3, kCarryOnly>), grid, block, 0, stream, p);
   } else if (p.vec_ok && p.head_dim == 64) {
-    hipLaunchKernelGGL((fwd_kernel<T, 64, true, 64, 2>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<T, 64, true, 64, 2, kCarryOnly>), grid, block, 0, stream, p);
   } else if (p.head_dim <= 64) {
-    hipLaunchKernelGGL((fwd_kernel<T, 64, false, 64, 2>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<T, 64, false, 64, 2, kCarryOnly>), grid, block, 0, stream, p);
   } else {
-    hipLaunchKernelGGL((fwd_kernel<T, 128, false, 64, 2>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<T, 128, false, 64, 2, kCarryOnly>), grid, block, 0, stream, p);
   }
   return hipGetLastError();
 }
 
 hipError_t launch_fwd(const FwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream) {
-  return dtype_is_f16 ? launch_fwd_t<_Float16>(p, max_tiles, stream)
-                      : launch_fwd_t<__bf16>(p, max_tiles, stream);
+  return dtype_is_f16 ? launch_fwd_t<_Float16, false>(p, max_tiles, stream)
+                      : launch_fwd_t<__bf16, false>(p, max_tiles, stream);
+}
+
+// The products the backward starts from, rebuilt from q and k alone (p.carry must be set; o, rem, row_stat, v unused).
+hipError_t launch_fwd_carry_only(const FwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream) {
+  return dtype_is_f16 ? launch_fwd_t<_Float16, true>(p, max_tiles, stream)
+                      : launch_fwd_t<__bf16, true>(p, max_tiles, stream);
 }
 
 }  // namespace sba

@@ -15,7 +15,7 @@ import torch
 from .utils import custom_op
 
 _LIB_NAME = "libsba.so"
-ABI_VERSION = 3          # SBA_VERSION of include/sba.h this binding mirrors
+ABI_VERSION = 4          # SBA_VERSION of include/sba.h this binding mirrors
 _lib = None
 # Optional ctypes array of hipEvent_t handed to the next calls as SbaArgs.trace_events (benchmarks only).
 TRACE_EVENTS = None
@@ -44,7 +44,7 @@ class SbaArgs(ctypes.Structure):
         ("d_o", SbaTensor), ("d_rem", SbaVector), ("dq", SbaTensor), ("dk", SbaTensor), ("dv", SbaTensor),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t), ("stream", ctypes.c_void_p),
         ("trace_events", ctypes.POINTER(ctypes.c_void_p)),
-        ("add_remainder", ctypes.c_int32), ("reserved0", ctypes.c_int32), ("carry_slots", ctypes.c_int64),
+        ("add_remainder", ctypes.c_int32), ("recompute_carry", ctypes.c_int32), ("carry_slots", ctypes.c_int64),
     ]
 
 
@@ -237,7 +237,10 @@ def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leadin
         a.row_stat = neg_log_acc.data_ptr() if neg_log_acc.numel() > 0 else None
         a.q, a.k, a.v, a.d_o, a.dq, a.dk, a.dv = (_tensor(t, fixed) for t in (q, k, v, do, dq, dk, dv))
         a.d_rem = _vector(drem, fixed)
-        a.carry = carry.data_ptr()
+        if carry.numel() > 0:
+            a.carry = carry.data_ptr()
+        else:
+            a.recompute_carry = 1        # the forward kept no products: rebuild them in the backward's workspace
         need = ctypes.c_size_t(0)
         _check(lib().sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(need), None), "sba_workspace_bytes")
         ws = torch.empty(need.value, dtype=torch.uint8, device=q.device)
@@ -249,8 +252,8 @@ def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leadin
 
 # The four launchers as out-parameter operators, registered for torch.compile the way the reference registers
 # its own (sb_varlen_fwd.py:453, sb_varlen_bwd.py:541, sb_attn/sb_fwd.py:175, sb_attn/sb_bwd.py:207).  ``carry``
-# replaces the reference's use of the saved ``neg_log_acc`` in the backward; an empty ``carry`` means "forward
-# only".
+# replaces the reference's use of the saved ``neg_log_acc`` in the backward; an empty ``carry`` means "do not
+# record it" in the forward and "rebuild it from q and k" in the backward.
 @custom_op("varlen_fwd", mutates_args={"o", "rem", "neg_log_acc", "carry"})
 def varlen_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor, cu_has_leading_zero: bool,
                max_seqlens: int, carry_slots: int, logit_scale: float, attend_current: bool, add_remainder: bool,
@@ -324,8 +327,13 @@ def forward(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, a
 def backward(do, drem, q, k, v, carry, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, attend_current,
              row_stat=None, add_remainder=False, carry_slots=0):
     """Launch the backward.  Returns (dq, dk, dv).  ``row_stat`` (the forward's third output) is needed when the
-    forward ran with ``add_remainder``.  Rows of a packed batch that belong to no sequence get zero gradients."""
+    forward ran with ``add_remainder``.  Rows of a packed batch that belong to no sequence get zero gradients.
+    ``carry=None``: the forward did not keep its products; the backward rebuilds them (16-bit dtypes only)."""
     _require_gpu(q, k, v, do, drem, carry)
+    if carry is None:
+        if q.dtype == torch.float32:
+            raise TypeError("save_carry=False is not available for fp32 inputs")
+        carry = torch.empty(0, dtype=torch.float32, device=q.device)
     fixed = cu_seqlens is None
     _same_dtype(q, k=k, v=v, do=do)
     do = rows_contiguous(do)

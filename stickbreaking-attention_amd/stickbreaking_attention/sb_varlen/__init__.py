@@ -19,8 +19,8 @@ class StickBreakingAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current, leading_zero=False, add_remainder=False,
-                carry_slots=0):
-        need_grad = any(ctx.needs_input_grad[:3])
+                carry_slots=0, save_carry=True):
+        need_grad = any(ctx.needs_input_grad[:3]) and (save_carry or q.dtype == torch.float32)   # fp32 always keeps them
         o, rem, row_stat, carry = _native.forward(q, k, v, cu_seqlens, leading_zero, max_seqlens, inv_temp,
                                                  attend_current, want_carry=need_grad, add_remainder=add_remainder,
                                                  carry_slots=carry_slots)
@@ -39,13 +39,16 @@ class StickBreakingAttention(torch.autograd.Function):
         dq, dk, dv = _native.backward(do, drem, q, k, v, carry, cu_seqlens, ctx.leading_zero,
                                       ctx.max_seqlens, ctx.logit_scale, ctx.attend_current,
                                       row_stat=row_stat, add_remainder=ctx.add_remainder, carry_slots=ctx.carry_slots)
-        return dq, dk, dv, None, None, None, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None, None, None
 
 
 def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, zero_start=True, attend_current=False,
-                   add_remainder=False):
+                   add_remainder=False, save_carry=True):
     """``add_remainder=True`` returns ``(o + rem[..., None] * v, rem)``: the combination every caller of the
-    reference forms from its outputs (tests/test_varlen.py:103), fused into the kernels' epilogues."""
+    reference forms from its outputs (tests/test_varlen.py:103), fused into the kernels' epilogues.
+    ``save_carry=False`` keeps only q, k, v between the forward and the backward, as the reference does, instead of
+    the per-(row, 32-key sub-tile) products (L^2 / 16 bytes per head and sequence); the backward rebuilds them with one
+    more kernel.  Gradients are bit-identical either way."""
     # The lengths are on the host when cu_seqlens was given as a CPU tensor, or after the one device-to-host copy that
     # stands in for the reference's `assert cu_seqlens[0] == 0` (sb_varlen/__init__.py:71-73, the same host sync).
     # They are then validated there and the carry buffer is sized exactly; a device-only cu_seqlens is validated by
@@ -66,7 +69,7 @@ def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, zero_st
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
     return StickBreakingAttention.apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current, bool(zero_start),
-                                        bool(add_remainder), carry_slots)
+                                        bool(add_remainder), carry_slots, bool(save_carry))
 
 
 def sb_attn_varlen_(q, k, v, inv_temp, cu_seqlens, max_seqlens, attend_current):

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol(native):
     lib = native.lib()
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.sba_version() == native.ABI_VERSION == 3
+    assert lib.sba_version() == native.ABI_VERSION == 4
     assert lib.sba_strerror(0) == b"ok"
     for code in range(-9, 0):
         assert lib.sba_strerror(code) not in (b"ok", b"unknown status")
@@ -131,8 +131,15 @@ def test_exact_carry_slots_shrink_the_buffers(native):
     assert native.carry_elems(H, T, len(lengths), 16384, False, exact) * 4 == carry_exact.value
     a.carry_slots = -1
     assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, None) == -6
-    a.carry_slots, a.reserved0 = 0, 1
+    a.carry_slots, a.recompute_carry = 0, 2
     assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, None) == -6
+    # rebuilding the products inside the backward moves the carry plane into the backward's workspace
+    a.carry_slots, a.recompute_carry = plan.carry_slots, 1
+    bwd_recompute = ctypes.c_size_t()
+    assert lib.sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(bwd_recompute), None) == 0
+    assert bwd_recompute.value == bwd_exact.value + carry_exact.value
+    a.dtype = 1
+    assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, None) == -2           # not for fp32
 
 
 def test_host_plan_rejects_what_the_scheduler_rejects(native):

@@ -55,12 +55,12 @@ def tol_check(name, got, ref, dtype, label, allowed_excess=0.0):
     return worst
 
 
-def run_varlen(q, k, v, cu, lengths, zero_start, attend_current, do, drem, scale=None, max_seqlens=True):
+def run_varlen(q, k, v, cu, lengths, zero_start, attend_current, do, drem, scale=None, max_seqlens=True, **options):
     from stickbreaking_attention import sb_attn_varlen
 
     q, k, v = (t.detach().clone().requires_grad_() for t in (q, k, v))
     o, rem = sb_attn_varlen(q, k, v, cu, max(lengths) if max_seqlens else None, inv_temp=scale, zero_start=zero_start,
-                            attend_current=attend_current)
+                            attend_current=attend_current, **options)
     outs = [o, rem]
     if do is not None:
         outs += list(torch.autograd.grad([o, rem], [q, k, v], [do, drem]))

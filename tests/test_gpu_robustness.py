@@ -102,6 +102,42 @@ def test_exact_carry_size_from_host_lengths(gpu_device, poisoned):
         sb_attn_varlen(*dev[:3], torch.tensor([5, 3, 10]), 10, zero_start=False)                # decreasing ends
 
 
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64), (torch.bfloat16, 72)])
+@pytest.mark.parametrize("attend_current", [False, True])
+def test_backward_that_rebuilds_the_forward_products(gpu_device, poisoned, dtype, D, attend_current):
+    # save_carry=False: nothing but q, k, v is kept between the passes (the reference's saved state, O(L)); the
+    # backward rebuilds the per-(row, sub-tile) products in its own workspace.  Same arithmetic, so the same bits,
+    # and parity with the oracle like every other path.
+    from stickbreaking_attention import sb_attn
+
+    lengths = [33, 500, 1, 129, 257, 64, 97]
+    host, dev, cu = small_case(2, D, lengths, dtype, seed=45)
+    ref = orc.varlen_stream(*host[:3], cu, attend_current=attend_current, do=host[3], drem=host[4], dtype=torch.float64)
+    for cu_arg in (cu.to(gpu_device), cu):                        # carry sized from the bound / exactly
+        kept = run_varlen(*dev[:3], cu_arg, lengths, False, attend_current, dev[3], dev[4])
+        rebuilt = run_varlen(*dev[:3], cu_arg, lengths, False, attend_current, dev[3], dev[4], save_carry=False)
+        for n, a, b, r in zip(NAMES, rebuilt, kept, ref):
+            assert torch.equal(a, b), f"{n}: rebuilt products give other bits than kept ones"
+            tol_check(n, a, r, dtype, f"rebuilt products {dtype} D={D}")
+    # with the remainder term fused, and in the fixed-length operator
+    kept = run_varlen(*dev[:3], cu.to(gpu_device), lengths, False, attend_current, dev[3], dev[4], add_remainder=True)
+    rebuilt = run_varlen(*dev[:3], cu.to(gpu_device), lengths, False, attend_current, dev[3], dev[4], add_remainder=True,
+                         save_carry=False)
+    for n, a, b in zip(NAMES, rebuilt, kept):
+        assert torch.equal(a, b), f"{n} (fused remainder)"
+    g = torch.Generator().manual_seed(46)
+    x = [torch.randn(2, 2, 300, D, generator=g).to(dtype).to(gpu_device) for _ in range(4)]
+    drem = torch.randn(2, 2, 300, generator=g).to(dtype).to(gpu_device)
+    grads = []
+    for save in (True, False):
+        q, k, v = (t.clone().requires_grad_() for t in x[:3])
+        o, rem = sb_attn(q, k, v, attend_current=attend_current, save_carry=save)
+        grads.append(torch.autograd.grad([o, rem], [q, k, v], [x[3], drem]))
+    torch.cuda.synchronize()
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("attend_current", [False, True])
 def test_token_major_producer_layouts_against_oracle(gpu_device, attend_current):
     """(T, H, D) packed and (B, L, H, D) fixed-length tensors permuted to the operators' layouts, as the reference's
