@@ -61,7 +61,7 @@ typedef enum SbaStatus {
                                base pointers that are multiples of 16 bytes select the fast kernels) */
   SBA_ERR_ALIGN = -5,       /* a tensor base pointer is not aligned to its element size */
   SBA_ERR_SHAPE = -6,       /* non-positive sizes, total_tokens > 2^30, a negative carry_slots or a flag outside {0, 1} */
-  SBA_ERR_WORKSPACE = -7,   /* workspace missing, not 256-byte aligned, or smaller than sba_workspace_bytes reports */
+  SBA_ERR_WORKSPACE = -7,   /* workspace missing, not 256-byte aligned, or too small (sba_bwd: smaller than one head needs) */
   SBA_ERR_LAUNCH = -8,      /* the HIP runtime rejected a launch (hipGetLastError) */
   SBA_ERR_TOO_LARGE = -9    /* sba_fwd_static: the tile schedule does not fit the library's static scratch */
 } SbaStatus;
@@ -203,6 +203,11 @@ int sba_fwd_static(const SbaArgs* args);
  * Replaces `_compileable_backward` (stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:541-640,
  * custom op "varlen_bwd") and (stickbreaking_attention/sb_attn/sb_bwd.py:207-296, custom op
  * "attn_bwd"), and the `locked_add` accumulation (sb_varlen_bwd.py:11-53).
+ * Workspace: bwd_bytes of sba_workspace_bytes runs all heads in one pass.  A smaller workspace is taken as a memory
+ * limit: the heads are independent, so the call takes them through in groups of as many as fit, one group after
+ * the other on the stream (same results).  The minimum is bwd_bytes of the same arguments with num_heads = 1;
+ * below that the call returns SBA_ERR_WORKSPACE before launching anything.  With several groups trace_events
+ * bracket the whole call but only the last group's dQ / dK/dV split.
  */
 int sba_bwd(const SbaArgs* args);
 

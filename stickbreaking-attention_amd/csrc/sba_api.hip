@@ -263,8 +263,13 @@ int sba_fwd_static(const SbaArgs* a) {
   return fwd_on(a, ws, kStaticScratchBytes, true);
 }
 
-int sba_bwd(const SbaArgs* a) {
-  if (!a) return SBA_ERR_NULL;
+}  // extern "C"
+
+namespace {
+
+// One pass of the backward over the heads `a` describes (all of them, or one group of a larger call: `stat_heads` is
+// the head count of the caller's row_stat array, `first`/`last` say which trace events this pass records).
+int bwd_pass(const SbaArgs* a, int64_t stat_heads, bool first, bool last) {
   Layout L;
   int st = plan(a, &L);
   if (st != SBA_OK) return st;
@@ -302,8 +307,9 @@ int sba_bwd(const SbaArgs* a) {
   p.attend_current = a->attend_current ? 1 : 0;
   p.add_rem = a->add_remainder ? 1 : 0;
   p.row_stat = a->row_stat;
-  p.stat_sb = fixed ? (int64_t)a->num_heads * a->total_tokens : 0;
+  p.stat_sb = fixed ? stat_heads * a->total_tokens : 0;
   p.stat_sh = a->total_tokens;
+  p.drem_sb = fixed ? (int64_t)a->num_heads * a->total_tokens : 0;
   p.drem_eff = (float*)(ws + L.off_drem);
   p.head_queue = (int32_t*)(ws + L.off_queue);
   p.max_tiles = (int32_t)L.max_q_tiles;
@@ -317,10 +323,10 @@ int sba_bwd(const SbaArgs* a) {
   const int key_tile = a->dtype == SBA_F32 ? kBlockK : sba::dkv_key_tile(p);
   if ((st = run_sched(a, ws, L, true, true, key_tile, stream)) != SBA_OK) return st;
   hipEvent_t* ev = (hipEvent_t*)a->trace_events;
-  if (ev && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  if (ev && first && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;
   if (a->dtype == SBA_F32) {
     if (sba::launch_bwd_f32(p, fixed ? a->num_seqs : 1, a->total_tokens, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
-    if (ev && (hipEventRecord(ev[1], stream) != hipSuccess || hipEventRecord(ev[2], stream) != hipSuccess)) return SBA_ERR_LAUNCH;
+    if (ev && last && (hipEventRecord(ev[1], stream) != hipSuccess || hipEventRecord(ev[2], stream) != hipSuccess)) return SBA_ERR_LAUNCH;
     return SBA_OK;
   }
   if (a->recompute_carry) {
@@ -345,9 +351,44 @@ int sba_bwd(const SbaArgs* a) {
     if (sba::launch_fwd_carry_only(f, a->dtype == SBA_F16, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
   }
   if (sba::launch_bwd_dq(p, a->dtype == SBA_F16, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
-  if (ev && hipEventRecord(ev[1], stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  if (ev && last && hipEventRecord(ev[1], stream) != hipSuccess) return SBA_ERR_LAUNCH;
   if (sba::launch_bwd_dkv(p, a->dtype == SBA_F16, (int)L.max_k_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
-  if (ev && hipEventRecord(ev[2], stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  if (ev && last && hipEventRecord(ev[2], stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  return SBA_OK;
+}
+
+
+}  // namespace
+
+extern "C" {
+
+int sba_bwd(const SbaArgs* a) {
+  if (!a) return SBA_ERR_NULL;
+  Layout L;
+  int st = plan(a, &L);
+  if (st != SBA_OK) return st;
+  if (a->workspace_bytes >= L.bwd_bytes || a->num_heads == 1) return bwd_pass(a, a->num_heads, true, true);
+  // A workspace smaller than the whole call needs: the heads are independent, so they go through in groups of as many
+  // as fit (the per-head planes dominate the workspace), one group after the other on the stream.
+  SbaArgs c = *a;
+  int64_t lo = 0, hi = a->num_heads;           // largest head count whose layout fits: plan() grows with num_heads
+  while (lo < hi) {
+    c.num_heads = (int32_t)((lo + hi + 1) / 2);
+    if (plan(&c, &L) == SBA_OK && L.bwd_bytes <= a->workspace_bytes) lo = c.num_heads; else hi = c.num_heads - 1;
+  }
+  if (lo < 1) return SBA_ERR_WORKSPACE;
+  const int64_t passes = cdiv(a->num_heads, lo), group = cdiv(a->num_heads, passes);
+  const size_t es = elem_size(a->dtype);
+  for (int64_t h0 = 0; h0 < a->num_heads; h0 += group) {
+    c = *a;
+    c.num_heads = (int32_t)(a->num_heads - h0 < group ? a->num_heads - h0 : group);
+    for (SbaTensor* t : {&c.q, &c.k, &c.v, &c.d_o, &c.dq, &c.dk, &c.dv})
+      if (t->ptr) t->ptr = (char*)t->ptr + h0 * t->stride_head * (int64_t)es;
+    if (c.d_rem.ptr) c.d_rem.ptr = (char*)c.d_rem.ptr + h0 * c.d_rem.stride_head * (int64_t)es;
+    if (c.carry) c.carry += h0 * L.carry_slots_per_head;          // slots per head do not depend on the head count
+    if (c.row_stat) c.row_stat += h0 * a->total_tokens;
+    if ((st = bwd_pass(&c, a->num_heads, h0 == 0, h0 + group >= a->num_heads)) != SBA_OK) return st;
+  }
   return SBA_OK;
 }
 

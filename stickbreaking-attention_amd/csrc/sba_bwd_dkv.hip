@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(BwdParams p) {
     } else {
       const bool diagonal = (j0 + kBlockK - 1) > (w_first - 1 + ac) || w_last >= L;
       // gradient of rem per row, as the dQ kernel left it (d_rem, plus d_o . v when the remainder term is fused)
-      const float drem = row_ok ? p.drem_eff[tile.seq_id * p.stat_sb + head * p.stat_sh + tok0 + qi] : 0.f;
+      const float drem = row_ok ? p.drem_eff[tile.seq_id * p.drem_sb + head * p.stat_sh + tok0 + qi] : 0.f;
       const float prod_in = carry[qi], prefix_in = prefix[qi];
       f32x16 s[2], dp[2];
 #pragma unroll
@@ -306,7 +306,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
 #pragma unroll
     for (int kk = 0; kk < kSteps; kk++) { kf[kk] = kf_next[kk]; vf[kk] = vf_next[kk]; }
     // Per-row scalars (drem, product above the sub-tile, C below it), fetched one step ahead.
-    const float* drem_eff = p.drem_eff + tile.seq_id * p.stat_sb + head * p.stat_sh + tok0;
+    const float* drem_eff = p.drem_eff + tile.seq_id * p.drem_sb + head * p.stat_sh + tok0;
     float n_drem = 0.f, n_prod = 1.f, n_prefix = 0.f;
     auto fetch_row_scalars = [&](int row0) {
       const int r = row0 + rg * 32 + col;
@@ -618,7 +618,7 @@ __global__ __launch_bounds__(kDkv4Threads) void bwd_dkv4_kernel(BwdParams p) {
                             carry_offset(4 * jt + g, n_qt) - (int64_t)kBlockQ * jt;      // + row
       const float* carry = p.carry + slot0;
       const float* prefix = p.prefix + slot0;
-      const float* drem_eff = p.drem_eff + tile.seq_id * p.stat_sb + head * p.stat_sh + tok0;
+      const float* drem_eff = p.drem_eff + tile.seq_id * p.drem_sb + head * p.stat_sh + tok0;
       // Per-row scalars (drem, product above the sub-tile, C below it), fetched two steps ahead: a step is shorter
       // than a global load.
       float n_drem = 0.f, n_prod = 1.f, n_prefix = 0.f, nn_drem = 0.f, nn_prod = 1.f, nn_prefix = 0.f;

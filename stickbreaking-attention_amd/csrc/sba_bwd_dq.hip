@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kThreads, KT == 32 ? 2 : 1) void bwd_dq_kernel(BwdP
     drem += dot + other_half(dot, half);
   }
   // The dK/dV kernel reads the gradient of rem back from this fp32 plane (one value per row).
-  if (half == 0 && row_ok) p.drem_eff[tile.seq_id * p.stat_sb + head * p.stat_sh + tok0 + qi] = drem;
+  if (half == 0 && row_ok) p.drem_eff[tile.seq_id * p.drem_sb + head * p.stat_sh + tok0 + qi] = drem;
   float prefix = 0.f;      // sum of g over the keys already swept (both half-waves hold the same value)
 
   const int last_row = min(q0 + kBlockQ, L) - 1;

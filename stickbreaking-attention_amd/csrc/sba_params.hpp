@@ -87,7 +87,8 @@ struct BwdParams {
   int64_t stat_sb, stat_sh;
   int32_t wgs_per_head;        // persistent dK/dV workgroups per head
   int32_t* head_queue;         // per head: next key tile not yet taken (beyond the first wgs_per_head), zero at launch
-  float* drem_eff;             // workspace, indexed like row_stat: the gradient of rem per row in fp32 (d_rem, plus
+  int64_t drem_sb;             // batch stride of drem_eff: the heads of THIS launch (row_stat's stride counts the caller's)
+  float* drem_eff;             // workspace, (B, heads, T) fp32: the gradient of rem per row in fp32 (d_rem, plus
                                // d_o . v when add_rem), written by the dQ kernel and read by the dK/dV kernel
   int32_t max_tiles;           // query-tile slots the dQ launch provides per head
   int64_t total_tokens;        // packed mode: rows of the token axis; rows no sequence covers are zero-filled

@@ -200,6 +200,17 @@ def carry_elems(num_heads: int, total_tokens: int, num_seqs: int, max_seqlen, fi
     return nbytes // 4
 
 
+# Upper limit in bytes for the backward's workspace (None: whatever the whole call needs).  With a limit the library
+# takes the heads through in groups that fit, one group after the other; together with ``save_carry=False`` this bounds
+# the memory of a long-context backward by the planes of one group of heads.
+BWD_WORKSPACE_LIMIT: Optional[int] = None
+
+
+def set_backward_workspace_limit(nbytes: Optional[int]):
+    global BWD_WORKSPACE_LIMIT
+    BWD_WORKSPACE_LIMIT = None if nbytes is None else int(nbytes)
+
+
 def _poison(t: torch.Tensor):
     t.view(torch.uint8).fill_(0xFF)          # every fp32 / 16-bit word becomes a NaN pattern, every int32 becomes -1
 
@@ -243,8 +254,15 @@ def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leadin
             a.recompute_carry = 1        # the forward kept no products: rebuild them in the backward's workspace
         need = ctypes.c_size_t(0)
         _check(lib().sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(need), None), "sba_workspace_bytes")
-        ws = torch.empty(need.value, dtype=torch.uint8, device=q.device)
-        a.workspace, a.workspace_bytes = ws.data_ptr(), need.value
+        nbytes = need.value
+        if BWD_WORKSPACE_LIMIT is not None and nbytes > BWD_WORKSPACE_LIMIT:
+            # the smallest workspace the library accepts is the one of a single head
+            heads, a.num_heads = a.num_heads, 1
+            _check(lib().sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(need), None), "sba_workspace_bytes")
+            a.num_heads = heads
+            nbytes = max(BWD_WORKSPACE_LIMIT, need.value)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), nbytes
         if POISON:
             _poison(ws)
         _check(lib().sba_bwd(ctypes.byref(a)), "sba_bwd")

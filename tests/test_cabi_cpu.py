@@ -140,6 +140,16 @@ def test_exact_carry_slots_shrink_the_buffers(native):
     assert bwd_recompute.value == bwd_exact.value + carry_exact.value
     a.dtype = 1
     assert lib.sba_workspace_bytes(ctypes.byref(a), None, None, None) == -2           # not for fp32
+    # a backward workspace smaller than the whole call is taken as a limit (the heads go through in groups), but it
+    # must hold at least one head: refused on the host, before anything is launched
+    a.dtype = 0
+    a.num_heads = 1
+    one_head = ctypes.c_size_t()
+    assert lib.sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(one_head), None) == 0
+    assert one_head.value < bwd_recompute.value / 16
+    a.num_heads = H
+    a.workspace, a.workspace_bytes = 256, one_head.value - 256          # never dereferenced: the size check comes first
+    assert lib.sba_bwd(ctypes.byref(a)) == -7
 
 
 def test_host_plan_rejects_what_the_scheduler_rejects(native):

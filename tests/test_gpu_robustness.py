@@ -138,6 +138,62 @@ def test_backward_that_rebuilds_the_forward_products(gpu_device, poisoned, dtype
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dtype,D,save_carry", [(torch.bfloat16, 128, False), (torch.bfloat16, 128, True),
+                                                 (torch.bfloat16, 64, False), (torch.float32, 32, True)])
+def test_backward_under_a_workspace_limit_goes_head_group_by_head_group(gpu_device, poisoned, dtype, D, save_carry):
+    # A backward workspace smaller than the whole call needs: the library processes as many heads at a time as fit.
+    # 5 heads under a limit that holds 2: passes of 2, 2 and 1 heads; same bits as the single pass.
+    from stickbreaking_attention import _native, sb_attn
+
+    lengths = [200, 33, 1, 385]
+    H = 5
+    host, dev, cu = small_case(H, D, lengths, dtype, seed=47)
+    options = dict(save_carry=save_carry, add_remainder=True)
+
+    def one_head_bytes():
+        a = _native._base_args(dev[0][:1], cu.to(gpu_device), False, max(lengths), 1.0, False)
+        a.recompute_carry = 0 if (save_carry or dtype == torch.float32) else 1
+        import ctypes
+        need = ctypes.c_size_t()
+        assert _native.lib().sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(need), None) == 0
+        return need.value
+
+    whole = run_varlen(*dev[:3], cu.to(gpu_device), lengths, False, False, dev[3], dev[4], **options)
+    g = torch.Generator().manual_seed(48)
+    x = [torch.randn(2, H, 300, D, generator=g).to(dtype).to(gpu_device) for _ in range(4)]
+    drem = torch.randn(2, H, 300, generator=g).to(dtype).to(gpu_device)
+
+    def fixed_grads():
+        q, k, v = (t.clone().requires_grad_() for t in x[:3])
+        o, rem = sb_attn(q, k, v, **options)
+        out = torch.autograd.grad([o, rem], [q, k, v], [x[3], drem])
+        torch.cuda.synchronize()
+        return out
+
+    whole_fixed = fixed_grads()
+    try:
+        _native.set_backward_workspace_limit(int(2.5 * one_head_bytes()))
+        limited = run_varlen(*dev[:3], cu.to(gpu_device), lengths, False, False, dev[3], dev[4], **options)
+        _native.set_backward_workspace_limit(1)                  # below one head: raised to the minimum, one head per pass
+        limited_fixed = fixed_grads()
+    finally:
+        _native.set_backward_workspace_limit(None)
+    for n, a, b in zip(NAMES, limited, whole):
+        if dtype == torch.float32 and n in ("dk", "dv"):          # summed with fp32 atomics on this path
+            assert torch.allclose(a, b, rtol=1e-5, atol=1e-5), n
+        else:
+            assert torch.equal(a, b), f"{n}: head groups give other bits than one pass"
+    for n, a, b in zip(NAMES[2:], limited_fixed, whole_fixed):
+        if dtype == torch.float32 and n in ("dk", "dv"):
+            assert torch.allclose(a, b, rtol=1e-5, atol=1e-5), n
+        else:
+            assert torch.equal(a, b), f"{n} (fixed length)"
+    ref = orc.varlen_stream(*host[:3], cu, do=host[3], drem=orc.remainder_drem(host[3], host[4], host[2]).float(),
+                            dtype=torch.float32)
+    for n, a, b in zip(NAMES, limited, orc.with_remainder(ref, host[2], host[3])):
+        tol_check(n, a, b, dtype, "head groups")
+
+
 @pytest.mark.parametrize("attend_current", [False, True])
 def test_token_major_producer_layouts_against_oracle(gpu_device, attend_current):
     """(T, H, D) packed and (B, L, H, D) fixed-length tensors permuted to the operators' layouts, as the reference's
@@ -241,3 +297,31 @@ def test_single_sequence_of_64k_tokens(gpu_device, poisoned):
     f32 = run_varlen(*(t.float() for t in dev[:3]), cu, [L], False, False, dev[3].float(), dev[4].float())
     for n, a, b in zip(NAMES, got, f32):
         tol_check(n, a, b.double().cpu(), torch.bfloat16, "64k vs fp32 path")
+
+
+def test_64k_tokens_four_heads_with_bounded_backward_memory(gpu_device, poisoned):
+    """The long-context configuration of the operator: nothing but q, k, v kept between the passes (save_carry=False)
+    and the backward's workspace capped at 600 MB, which holds the two per-(row, sub-tile) planes of ONE head at 65536
+    tokens (2 x 269 MB) -- the heads go through one at a time.  Same bits as the default mode, which holds 8 planes
+    (4 saved by the forward, 4 in the workspace) for the same call."""
+    from stickbreaking_attention import _native
+
+    L, D, H = 65536, 128, 4
+    g = torch.Generator().manual_seed(62)
+    q, k, v, do = (torch.randn(H, L, D, generator=g).bfloat16().to(gpu_device) for _ in range(4))
+    drem = torch.randn(H, L, generator=g).bfloat16().to(gpu_device)
+    cu = torch.tensor([L], dtype=torch.int32)
+    default = run_varlen(q, k, v, cu, [L], False, False, do, drem)
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    try:
+        _native.set_backward_workspace_limit(600 << 20)
+        bounded = run_varlen(q, k, v, cu, [L], False, False, do, drem, save_carry=False)
+    finally:
+        _native.set_backward_workspace_limit(None)
+    peak = torch.cuda.max_memory_allocated() - before
+    for n, a, b in zip(NAMES, bounded, default):
+        assert torch.equal(a, b), n
+    # inputs' clones, outputs, gradients (about 0.45 GB) + the 600 MB workspace; the default mode needs 2.1 GB of planes
+    assert peak < 1200 << 20, f"peak {peak >> 20} MiB"
