@@ -317,6 +317,23 @@ def test_config3_full_size(gpu_device):
     assert torch.equal(o[0], got[0][:, s0:s0 + n]) and torch.equal(rem[0], got[1][:, s0:s0 + n])
 
 
+def test_config3_shape_in_f16_with_the_current_token_and_rebuilt_products(gpu_device):
+    # The benchmark shape once more through the paths the bf16 run does not take: fp16 storage, attend_current=True,
+    # and a backward that rebuilds the forward's products (bit-identical to the one that was handed them).
+    inp = bench.make_inputs("c3", gpu_device)
+    lengths = inp["lengths"]
+    dev = [inp[n].to(torch.float16) for n in ("q", "k", "v", "do", "drem")]
+    kept = run_varlen(*dev[:3], inp["cu"], lengths, False, True, dev[3], dev[4])
+    rebuilt = run_varlen(*dev[:3], inp["cu"], lengths, False, True, dev[3], dev[4], save_carry=False)
+    for n, a, b in zip(NAMES, rebuilt, kept):
+        assert torch.equal(a, b), n
+    heads = [3, 28]
+    host = [t[heads].cpu() for t in dev]
+    ref = orc.varlen_stream(*host[:3], inp["cu"].cpu(), attend_current=True, do=host[3], drem=host[4], dtype=torch.float64)
+    for n, a, b in zip(NAMES, kept, ref):
+        tol_check(n, a[heads], b, torch.float16, "c3 f16 attend_current")
+
+
 def test_config4_fixed_full_size(gpu_device):
     from stickbreaking_attention import sb_attn
 
