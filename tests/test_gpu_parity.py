@@ -386,6 +386,22 @@ def test_config5_adversarial_long_sequence(config5_run):
     _check_against_floor("c5 long sequence", [t[h, short_T:] for t in got], floor, exact)
 
 
+def test_config5_with_rebuilt_products_in_head_groups(gpu_device, config5_run):
+    # the adversarial batch once more with nothing kept between the passes and the backward's workspace capped at 300 MB
+    # (the planes of 32 heads need 1.07 GB here): same bits as the default run
+    from stickbreaking_attention import _native
+
+    lengths, host, got = config5_run
+    inp = bench.make_inputs("c5", gpu_device)
+    try:
+        _native.set_backward_workspace_limit(300 << 20)
+        again = run_varlen(inp["q"], inp["k"], inp["v"], inp["cu"], lengths, True, False, inp["do"], inp["drem"], save_carry=False)
+    finally:
+        _native.set_backward_workspace_limit(None)
+    for n, a, b in zip(NAMES, again, got):
+        assert torch.equal(a.cpu(), b), n
+
+
 def test_forward_without_grad_skips_carry(gpu_device):
     from stickbreaking_attention import _native
 
