@@ -39,13 +39,15 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 4
+#define SBA_VERSION 5
 
 /* Scheduler status word: int32 at this byte offset of the workspace, valid after the stream has run. */
 #define SBA_STATUS_OFFSET 8
 #define SBA_SCHED_OK 0
 #define SBA_SCHED_BAD_CU_SEQLENS 1
 #define SBA_SCHED_CARRY_TOO_SMALL 2
+#define SBA_CHAIN_TIMEOUT 3        /* one-kernel backward: a workgroup gave up waiting for the key tile below its own */
+#define SBA_CHAIN_XCD_MISMATCH 4   /* one-kernel backward: the workgroups of a head did not share an XCD */
 
 /* Size of the static device scratch behind sba_fwd_static. */
 #define SBA_STATIC_SCRATCH_BYTES ((size_t)1 << 20)
@@ -131,6 +133,12 @@ typedef struct SbaArgs {
                                   need of a ragged batch; a caller that knows the lengths on the host passes
                                   SbaPlan.carry_slots from sba_plan_host for the exact size.  Must be the same in the
                                   forward, the backward and sba_workspace_bytes. */
+  int32_t backward_kernels;    /* 0 or 1: sba_bwd runs a dQ kernel and a dK/dV kernel.  2: where it applies (head_dim 128,
+                                  16-bit, 16-byte aligned rows, a head count that is a multiple of 8, no add_remainder)
+                                  ONE kernel in which the key tiles of a sequence hand the row prefix sums and the partial
+                                  dQ to each other, the two kernels otherwise.  Must be the same in sba_workspace_bytes
+                                  and sba_bwd. */
+  int32_t reserved0;
 } SbaArgs;
 
 /* What the device scheduler will derive from cu_seqlens, computed on the host from a host copy. */

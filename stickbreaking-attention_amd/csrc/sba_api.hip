@@ -13,6 +13,8 @@ hipError_t launch_fwd_carry_only(const FwdParams& p, int dtype_is_f16, int max_t
 hipError_t launch_bwd_dq(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
 hipError_t launch_bwd_dkv(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
 int dkv_key_tile(const BwdParams& p);
+bool chain_supported(const BwdParams& p);
+hipError_t launch_bwd_chain(const BwdParams& p, int dtype_is_f16, int max_tiles, hipStream_t stream);
 hipError_t launch_fwd_f32(const FwdParams& p, int max_tiles, hipStream_t stream);
 hipError_t launch_bwd_f32(const BwdParams& p, int batches, int64_t tokens, int max_q_tiles, hipStream_t stream);
 }  // namespace sba
@@ -29,6 +31,10 @@ struct Layout {
   int64_t max_q_tiles, max_k_tiles, carry_slots_per_head;
   size_t off_counts, off_q_tiles, off_k_tiles, off_carry_base, off_prefix, off_drem, off_queue, off_carry;
   size_t fwd_bytes, bwd_bytes, carry_bytes;
+  // One-kernel backward: its buffers share the prefix plane's region (only one of the two backwards runs).
+  int64_t chain_rows;                       // rows per head
+  size_t off_chain_zero, chain_zero_bytes;  // {C, tag} per row, the flags and the heads' XCC ids: cleared by every launch
+  size_t off_chain_c, off_chain_flags, off_chain_xcc, off_chain_dq;
 };
 
 int plan(const SbaArgs* a, Layout* out) {
@@ -37,6 +43,7 @@ int plan(const SbaArgs* a, Layout* out) {
   if (a->dtype != SBA_BF16 && a->dtype != SBA_F16 && a->dtype != SBA_F32) return SBA_ERR_DTYPE;
   if (a->total_tokens > (int64_t)1 << 30) return SBA_ERR_SHAPE;
   if ((a->recompute_carry != 0 && a->recompute_carry != 1) || a->carry_slots < 0) return SBA_ERR_SHAPE;
+  if (a->backward_kernels < 0 || a->backward_kernels > 2) return SBA_ERR_SHAPE;
   if (a->recompute_carry && a->dtype == SBA_F32) return SBA_ERR_DTYPE;      // the fp32 path always keeps its products
   Layout L{};
   const int64_t T = a->total_tokens, B = a->num_seqs;
@@ -61,7 +68,19 @@ int plan(const SbaArgs* a, Layout* out) {
   L.fwd_bytes = off;
   L.off_k_tiles = off;     off = align_up(off + (size_t)L.max_k_tiles * sizeof(sba::Tile), 256);
   L.carry_bytes = align_up((size_t)L.carry_slots_per_head * a->num_heads * sizeof(float), 256);
-  L.off_prefix = off;      off += L.carry_bytes;
+  size_t chain_bytes = 0;
+  L.chain_rows = fixed ? B * T : T;
+  if (a->dtype != SBA_F32 && a->head_dim == 128 && (a->num_heads & 7) == 0 && !a->add_remainder && a->backward_kernels == 2) {
+    size_t c = off;
+    L.off_chain_zero = c;
+    L.off_chain_c = c;      c = align_up(c + (size_t)a->num_heads * L.chain_rows * 8, 256);
+    L.off_chain_flags = c;  c = align_up(c + (size_t)a->num_heads * L.max_k_tiles * 32, 256);
+    L.off_chain_xcc = c;    c = align_up(c + (size_t)a->num_heads * 4, 256);
+    L.chain_zero_bytes = c - L.off_chain_zero;
+    L.off_chain_dq = c;     c += (size_t)a->num_heads * L.chain_rows * 128 * sizeof(float);
+    chain_bytes = align_up(c - off, 256);
+  }
+  L.off_prefix = off;      off += L.carry_bytes > chain_bytes ? L.carry_bytes : chain_bytes;
   // d_rem + d_o . v per row (fp32), used when the remainder term is fused
   L.off_drem = off;        off = align_up(off + (size_t)a->num_heads * (size_t)T * (fixed ? (size_t)B : 1) * sizeof(float), 256);
   L.off_queue = off;       off = align_up(off + (size_t)a->num_heads * sizeof(int32_t), 256);      // per-head tile cursors
@@ -92,8 +111,13 @@ int check_tensor(const SbaTensor& t, bool required, bool fixed) {
 sba::TensorRef ref(const SbaTensor& t, bool fixed) { return sba::TensorRef{t.ptr, fixed ? t.stride_batch : 0, t.stride_head, t.stride_token}; }
 sba::VectorRef vref(const SbaVector& t, bool fixed) { return sba::VectorRef{t.ptr, fixed ? t.stride_batch : 0, t.stride_head, t.stride_token}; }
 
-int run_sched(const SbaArgs* a, char* ws, const Layout& L, bool want_key_tiles, bool want_carry_base, int key_tile, hipStream_t stream) {
+int run_sched(const SbaArgs* a, char* ws, const Layout& L, bool want_key_tiles, bool want_carry_base, int key_tile, hipStream_t stream,
+              bool clear_chain = false) {
   sba::SchedParams sp{};
+  if (clear_chain) {
+    sp.zero_fill = (uint32_t*)(ws + L.off_chain_zero);
+    sp.zero_bytes = (int64_t)L.chain_zero_bytes;
+  }
   sp.cu = a->cu_seqlens;
   sp.cu_is_int64 = a->cu_is_int64;
   sp.cu_has_leading_zero = a->cu_has_leading_zero;
@@ -319,9 +343,21 @@ int bwd_pass(const SbaArgs* a, int64_t stat_heads, bool first, bool last) {
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
     if (t->ptr) v16 = v16 && vec16(*t, es, fixed, max_rows);
   p.vec_ok = v16 ? 1 : 0;
+  // One kernel (the key tiles of a sequence hand C and partial dQ to each other) where it applies, else dQ then dK/dV.
+  const bool chain = a->dtype != SBA_F32 && L.chain_zero_bytes > 0 && sba::chain_supported(p);
+  if (chain) {
+    p.chain_c = (uint32_t*)(ws + L.off_chain_c);
+    p.chain_flags = (int32_t*)(ws + L.off_chain_flags);
+    p.chain_head_xcc = (int32_t*)(ws + L.off_chain_xcc);
+    p.chain_dq = (float*)(ws + L.off_chain_dq);
+    p.status = (int32_t*)(ws + L.off_counts) + sba::kCountStatus;
+    p.chain_rows = L.chain_rows;
+    p.chain_sb = fixed ? a->total_tokens : 0;
+    p.chain_tile_cap = (int32_t)L.max_k_tiles;
+  }
   // The key-tile list is built for the dK/dV kernel that will run (the fp32 kernels do not use it).
   const int key_tile = a->dtype == SBA_F32 ? kBlockK : sba::dkv_key_tile(p);
-  if ((st = run_sched(a, ws, L, true, true, key_tile, stream)) != SBA_OK) return st;
+  if ((st = run_sched(a, ws, L, true, true, key_tile, stream, chain)) != SBA_OK) return st;
   hipEvent_t* ev = (hipEvent_t*)a->trace_events;
   if (ev && first && hipEventRecord(ev[0], stream) != hipSuccess) return SBA_ERR_LAUNCH;
   if (a->dtype == SBA_F32) {
@@ -349,6 +385,12 @@ int bwd_pass(const SbaArgs* a, int64_t stat_heads, bool first, bool last) {
     for (const SbaTensor* t : {&a->q, &a->k}) fv16 = fv16 && vec16(*t, es, fixed, max_rows);
     f.vec_ok = fv16 ? 1 : 0;
     if (sba::launch_fwd_carry_only(f, a->dtype == SBA_F16, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
+  }
+  if (chain) {
+    if (ev && last && hipEventRecord(ev[1], stream) != hipSuccess) return SBA_ERR_LAUNCH;
+    if (sba::launch_bwd_chain(p, a->dtype == SBA_F16, (int)L.max_k_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
+    if (ev && last && hipEventRecord(ev[2], stream) != hipSuccess) return SBA_ERR_LAUNCH;
+    return SBA_OK;
   }
   if (sba::launch_bwd_dq(p, a->dtype == SBA_F16, (int)L.max_q_tiles, stream) != hipSuccess) return SBA_ERR_LAUNCH;
   if (ev && last && hipEventRecord(ev[1], stream) != hipSuccess) return SBA_ERR_LAUNCH;

@@ -25,7 +25,7 @@ struct Tile {
 // Slots of the scheduler's `counts` array.
 enum : int { kCountQ = 0, kCountK = 1, kCountStatus = 2, kCountCovered = 3 };
 // Values of counts[kCountStatus].
-enum : int { kSchedOk = 0, kSchedBadCu = 1, kSchedCarryOverflow = 2 };
+enum : int { kSchedOk = 0, kSchedBadCu = 1, kSchedCarryOverflow = 2, kSchedChainTimeout = 3, kSchedChainXcd = 4 };
 
 struct SchedParams {
   const void* cu;          // NULL: fixed-length mode
@@ -45,6 +45,8 @@ struct SchedParams {
   int32_t* head_queue;     // backward: per-head cursor into the key-tile list, reset to 0 here
   int32_t num_heads;
   int32_t key_tile;        // keys per key tile (a multiple of 32; what the dK/dV kernel that will run sweeps)
+  uint32_t* zero_fill;     // optional: 16-byte aligned region cleared by the launch (the one-kernel backward's flags
+  int64_t zero_bytes;      // and tags start every call at zero), a multiple of 16 bytes
 };
 
 struct FwdParams {
@@ -92,6 +94,15 @@ struct BwdParams {
                                // d_o . v when add_rem), written by the dQ kernel and read by the dK/dV kernel
   int32_t max_tiles;           // query-tile slots the dQ launch provides per head
   int64_t total_tokens;        // packed mode: rows of the token axis; rows no sequence covers are zero-filled
+  // One-kernel backward (sba_bwd_chain.hip): what the key tiles of a (head, sequence) hand to each other.
+  float* chain_dq;             // [head][row][128] fp32: partial dQ of a row over the key tiles below the reader
+  uint32_t* chain_c;           // [head][row] {fp32 C below the reader's tile, tag = index of the reader's tile}
+  int32_t* chain_flags;        // [head][key tile slot][8]: per consumer wave, row blocks whose partial dQ is complete
+  int32_t* chain_head_xcc;     // [head]: XCC id + 1 of the head's workgroups (0 = none yet)
+  int32_t* status;             // the scheduler's status word; the kernel raises it when a wait runs out
+  int64_t chain_rows;          // rows per head in chain_dq / chain_c
+  int64_t chain_sb;            // fixed-length mode: rows per batch element (0 in packed mode)
+  int32_t chain_tile_cap;      // key-tile slots per head in chain_flags
 };
 
 // One sequence's token range from cu_seqlens (cumulative sequence ends, optionally preceded by a 0).  Returns false

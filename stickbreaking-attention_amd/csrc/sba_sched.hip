@@ -45,6 +45,13 @@ __device__ void descending_offsets(int* bins, int* scratch) {
 }
 
 __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
+  if (blockIdx.x > 0) {      // helper workgroups: clear the region the launch was asked to clear
+    const int64_t n16 = p.zero_bytes / 16, per = (n16 + gridDim.x - 2) / (gridDim.x - 1);
+    const int64_t a = per * (blockIdx.x - 1), b = a + per < n16 ? a + per : n16;
+    u32x4* z = reinterpret_cast<u32x4*>(p.zero_fill);
+    for (int64_t i = a + threadIdx.x; i < b; i += kSchedThreads) z[i] = u32x4{0u, 0u, 0u, 0u};
+    return;
+  }
   __shared__ int qbins[kBins];
   __shared__ int kbins[kBins];
   __shared__ int scratch[kSchedThreads];
@@ -150,7 +157,13 @@ __global__ __launch_bounds__(kSchedThreads) void sched_kernel(SchedParams p) {
 }
 
 hipError_t launch_sched(const SchedParams& p, hipStream_t stream) {
-  hipLaunchKernelGGL(sched_kernel, dim3(1), dim3(kSchedThreads), 0, stream, p);
+  // One workgroup schedules; with a region to clear, one more per 256 KiB of it (at most 64) clears alongside.
+  int helpers = 0;
+  if (p.zero_fill && p.zero_bytes > 0) {
+    helpers = (int)((p.zero_bytes + (256 << 10) - 1) / (256 << 10));
+    if (helpers > 64) helpers = 64;
+  }
+  hipLaunchKernelGGL(sched_kernel, dim3(1 + helpers), dim3(kSchedThreads), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -15,7 +15,7 @@ import torch
 from .utils import custom_op
 
 _LIB_NAME = "libsba.so"
-ABI_VERSION = 4          # SBA_VERSION of include/sba.h this binding mirrors
+ABI_VERSION = 5          # SBA_VERSION of include/sba.h this binding mirrors
 _lib = None
 # Optional ctypes array of hipEvent_t handed to the next calls as SbaArgs.trace_events (benchmarks only).
 TRACE_EVENTS = None
@@ -45,6 +45,7 @@ class SbaArgs(ctypes.Structure):
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t), ("stream", ctypes.c_void_p),
         ("trace_events", ctypes.POINTER(ctypes.c_void_p)),
         ("add_remainder", ctypes.c_int32), ("recompute_carry", ctypes.c_int32), ("carry_slots", ctypes.c_int64),
+        ("backward_kernels", ctypes.c_int32), ("reserved0", ctypes.c_int32),
     ]
 
 
@@ -59,6 +60,23 @@ STATUS_OFFSET = 8        # SBA_STATUS_OFFSET: the scheduler's status word inside
 # Debugging aid for the tests: fill the carry buffer and the workspaces with NaN bit patterns before every launch,
 # so that a kernel reading a slot nobody wrote shows up as NaN instead of passing on whatever the allocator returned.
 POISON = os.environ.get("SBA_DEBUG_POISON", "0") == "1"
+# Read the scheduler's status word back after every launch (one device-to-host copy and a synchronisation per call)
+# and raise on a schedule the device refused.  Without it a bad ``cu_seqlens`` that only exists on the device yields
+# all-zero outputs and gradients and no error.
+DEBUG_CHECK = os.environ.get("SBA_DEBUG_CHECK", "0") == "1"
+# SbaArgs.backward_kernels: 0 / 1 = dQ then dK/dV, 2 = one chained kernel where it applies.
+BACKWARD_KERNELS = int(os.environ.get("SBA_BACKWARD_KERNELS", "0"))
+_STATUS_TEXT = {1: "cu_seqlens is not a non-decreasing sequence within [0, total_tokens] (or its leading entry is not 0)",
+                2: "the carry buffer is too small for these sequence lengths (max_seqlens understated?)",
+                3: "one-kernel backward: a workgroup gave up waiting for the key tile below its own",
+                4: "one-kernel backward: the workgroups of a head did not share an XCD"}
+
+
+def check_status(ws: torch.Tensor, what: str):
+    """Raise if the device-side scheduler (or the chained backward) left a non-zero status word in ``ws``."""
+    status = int(ws[STATUS_OFFSET:STATUS_OFFSET + 4].view(torch.int32).item())
+    if status != 0:
+        raise ValueError(f"{what}: {_STATUS_TEXT.get(status, 'status %d' % status)}; outputs of this call are not valid")
 
 
 def library_path() -> str:
@@ -169,6 +187,7 @@ def _base_args(q, cu_seqlens, cu_has_leading_zero, max_seqlen, logit_scale, atte
     a.logit_scale = float(logit_scale)
     a.attend_current = 1 if attend_current else 0
     a.stream = torch.cuda.current_stream(q.device).cuda_stream
+    a.backward_kernels = BACKWARD_KERNELS
     if TRACE_EVENTS is not None:
         a.trace_events = ctypes.cast(TRACE_EVENTS, ctypes.POINTER(ctypes.c_void_p))
     return a
@@ -237,6 +256,8 @@ def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, carry_slot
                 raise RuntimeError(f"carry buffer too small: {carry.numel() * 4} < {need_carry.value} bytes")
             a.carry = carry.data_ptr()
         _check(lib().sba_fwd(ctypes.byref(a)), "sba_fwd")
+        if DEBUG_CHECK:
+            check_status(ws, "sba_fwd")
 
 
 def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leading_zero, max_seqlen, carry_slots, logit_scale,
@@ -266,6 +287,8 @@ def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leadin
         if POISON:
             _poison(ws)
         _check(lib().sba_bwd(ctypes.byref(a)), "sba_bwd")
+        if DEBUG_CHECK:
+            check_status(ws, "sba_bwd")
 
 
 # The four launchers as out-parameter operators, registered for torch.compile the way the reference registers

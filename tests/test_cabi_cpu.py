@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol(native):
     lib = native.lib()
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.sba_version() == native.ABI_VERSION == 4
+    assert lib.sba_version() == native.ABI_VERSION == 5
     assert lib.sba_strerror(0) == b"ok"
     for code in range(-9, 0):
         assert lib.sba_strerror(code) not in (b"ok", b"unknown status")
@@ -43,10 +43,10 @@ def test_library_exports_every_declared_symbol(native):
 
 def test_struct_layout_matches_header(native, tmp_path):
     src = tmp_path / "sz.c"
-    src.write_text('#include "sba.h"\n#include <stdio.h>\n#include <stddef.h>\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu\\n", '
+    src.write_text('#include "sba.h"\n#include <stdio.h>\n#include <stddef.h>\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n", '
                    "sizeof(SbaArgs), offsetof(SbaArgs,q), offsetof(SbaArgs,carry), offsetof(SbaArgs,d_o), "
                    "offsetof(SbaArgs,workspace), offsetof(SbaArgs,trace_events), offsetof(SbaArgs,carry_slots), "
-                   "sizeof(SbaPlan), offsetof(SbaPlan,pairs));}\n")
+                   "offsetof(SbaArgs,backward_kernels), sizeof(SbaPlan), offsetof(SbaPlan,pairs));}\n")
     exe = tmp_path / "sz"
     import subprocess
 
@@ -55,7 +55,7 @@ def test_struct_layout_matches_header(native, tmp_path):
     A = native.SbaArgs
     P = native.SbaPlan
     assert got == [ctypes.sizeof(A), A.q.offset, A.carry.offset, A.d_o.offset, A.workspace.offset, A.trace_events.offset,
-                   A.carry_slots.offset, ctypes.sizeof(P), P.pairs.offset]
+                   A.carry_slots.offset, A.backward_kernels.offset, ctypes.sizeof(P), P.pairs.offset]
 
 
 def _args(native, H, D, T, B, varlen=True, max_seqlen=0, dtype=0):
