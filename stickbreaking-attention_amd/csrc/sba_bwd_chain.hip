@@ -140,6 +140,25 @@ __device__ __forceinline__ void ch_landed4(u32x4& a, u32x4& b, u32x4& c, u32x4& 
 __device__ __forceinline__ u32x4 ch_join(const u32x2& lo, const u32x2& hi) { return u32x4{lo[0], lo[1], hi[0], hi[1]}; }
 
 // A load that bypasses the vector L1 (sc1): what another workgroup of this XCD stored and completed is seen.
+// Loads of the chain by the consumer waves, as inline assembly: the wave waits for exactly these (loads return in
+// order) and not for the younger row requests, which the compiler's own wait counts cannot express across the
+// branches in between.  sc1: served by the L2, never by this compute unit's vector cache.
+template <int kOff>
+__device__ __forceinline__ void ch_chain_load(u32x4& v, int voff, u32x4 desc, int soff) {
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4 sc1" : "=v"(v) : "v"(voff), "s"(desc), "s"(soff), "n"(kOff) : "memory");
+}
+__device__ __forceinline__ void ch_flag_request(int& v, const int32_t* f) {
+  asm volatile("global_load_dword %0, %1, %2 sc1" : "=v"(v) : "v"(0), "s"(f) : "memory");
+}
+// Wait until at most kLeft vector memory operations of this wave are outstanding.
+// Placed after the wait for the loads above: from here on the compiler may read their registers.  (One statement for
+// all paths: two of these in the arms of a branch make the compiler merge their results with register copies placed
+// in front of the waits.)
+__device__ __forceinline__ void ch_chain_landed(u32x4 (&c)[4], int& flag) {
+  asm volatile("" : "+v"(c[0]), "+v"(c[1]), "+v"(c[2]), "+v"(c[3]), "+v"(flag) :: "memory");
+}
+template <int kLeft>
+__device__ __forceinline__ void ch_vm_wait() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kLeft) : "memory"); }
 __device__ __forceinline__ int ch_load_flag(const int32_t* f) {
   return __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -554,10 +573,12 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
       bool have_next = false;
       int32_t* const my_flag = p.chain_flags + ((int64_t)head * p.chain_tile_cap + slot_idx) * 8 + c;
       const int32_t* const pred_flag = my_flag - 8;
-      int flag_seen = 0, flag_pre = 0;                       // the tile below's count for this wave's columns, as last read
+      int flag_seen = 0;                                     // the tile below's count for this wave's columns, as last read
       // dQ partial sums of this sequence's rows (fp32, [row][128]) and the dq output, addressed per sequence.
       const __amdgpu_buffer_rsrc_t dqc_rs = __builtin_amdgcn_make_buffer_rsrc(
           (void*)(p.chain_dq + ((int64_t)head * p.chain_rows + f.crow) * DH), 0, L * DH * 4, 0x00020000);
+      const uint64_t dqc_addr = (uint64_t)(p.chain_dq + ((int64_t)head * p.chain_rows + f.crow) * DH);
+      const u32x4 dqc_desc = {(uint32_t)dqc_addr, (uint32_t)(dqc_addr >> 32) & 0xffffu, (uint32_t)(L * DH * 4), 0x00020000u};
       const RowSink<T> dq_sink = make_row_sink<T>((T*)p.dq.ptr + tile.seq_id * p.dq.sb + head * p.dq.sh + f.tok0 * p.dq.st, p.dq.st, L, DH);
       const int dqc_voff = col * (DH * 4) + (32 * c + 4 * half) * 4;
       const int dq_voff = col * dq_sink.stride_bytes + (32 * c + 4 * half) * 2;
@@ -565,36 +586,7 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
       for (int s = 0; s < S; ++s) {
         // ---- top of the slot: everything this wave has in flight completes, then it is published ---------------
         CH_T(6)
-        __builtin_amdgcn_s_waitcnt(0x0F70);
         CH_T(0)
-        if (pub_flag) {
-          if (lane == 0) __hip_atomic_store(pub_flag, pub_count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          pub_flag = nullptr;
-        }
-        // The next tile is claimed late and in three slots: the cursor, then the tile record, then LDS.
-        if (c == 3) {
-          if (s == f.a) { if (lane == 0) claim_v = atomicAdd(p.head_queue + head, 1); }
-          else if (s == f.a + 1) {
-            claim_v = __builtin_amdgcn_readfirstlane(claim_v);
-            if (claim_v < n_tiles && lane < 6) rec_w = reinterpret_cast<const uint32_t*>(p.k_tiles + claim_v)[lane];
-          } else if (s == f.a + 2) {
-            if (lane < 6) next_lds[lane] = (int)rec_w;
-            if (lane == 0) next_lds[8] = claim_v;
-          }
-        }
-        if (s == f.a + 3) {
-          const int ns = __builtin_amdgcn_readfirstlane(next_lds[8]);
-          have_next = ns < n_tiles;
-          if (have_next) {
-            next_tile.seq_start = __builtin_amdgcn_readfirstlane(next_lds[0]);
-            next_tile.seq_len = __builtin_amdgcn_readfirstlane(next_lds[1]);
-            next_tile.origin = __builtin_amdgcn_readfirstlane(next_lds[2]);
-            next_tile.seq_id = __builtin_amdgcn_readfirstlane(next_lds[3]);
-            const uint32_t lo = __builtin_amdgcn_readfirstlane(next_lds[4]), hi = __builtin_amdgcn_readfirstlane(next_lds[5]);
-            next_tile.carry_base = (int64_t)(((uint64_t)hi << 32) | lo);
-            slot_idx = ns;                                   // used for the flags of the next tile (read at its start)
-          }
-        }
         if (s == 0) {
           // K^T of this tile for the dQ contraction, through the wave's scratch: [32 keys][32 columns] at a time,
           // gathered down the keys by the transpose read.  The previous tile's results leave first (same scratch).
@@ -633,42 +625,42 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
         const int qz0 = kChRows * (f.nb - 1 - kz);
         const bool final_rows = kz >= n - 4;                 // rows of the tile's own 128-row block: dq leaves
         const bool chain_in = has_z && J > 0 && !(kChX & 2);
-        f32x4 cdq[4];                                        // the partial dQ from the tiles below
-        auto load_chain_in = [&]() {
-          // (must be issued after the flag has been seen: the flag load is relaxed, so the compiler is told here;
-          // the hardware issues this wave's loads in program order)
-          asm volatile("" ::: "memory");
-#pragma unroll
-          for (int a4 = 0; a4 < 4; a4++)     // (whole-vector bit casts: a bit cast of one element of a vector reads element 0)
-            cdq[a4] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(dqc_rs, dqc_voff + 32 * a4, qz0 * (DH * 4), kAuxSc1));
-        };
-        // The count the tile below has published for this wave's columns was requested at the end of the previous slot;
-        // if that was too early, it is requested again here and looked at after the contraction.
+        // The partial dQ from the tiles below goes straight into the accumulator of this slot's dQ MFMAs.  The count the
+        // tile below has published for this wave's columns was requested at the end of the previous slot; if that was
+        // too early the wave polls here.  (Whole-vector bit casts: a bit cast of one element of a vector reads element 0.)
+        const bool do_dq = has_z && !(kChX & 4);
+        const bool take_in = do_dq && chain_in;
+        u32x4 cin[4];
         int flag_v = 0;
-        bool flag_asked = false, cdq_loaded = false;
-        if (chain_in) {
-          if (flag_seen < kz + 1) flag_seen = flag_pre;
-          if ((kChX & 1) || aborted || flag_seen >= kz + 1) { load_chain_in(); cdq_loaded = true; }
-          else { flag_v = ch_load_flag(pred_flag); flag_asked = true; }
+        if (take_in) {
+          if (!(kChX & 1) && !aborted && flag_seen < kz + 1) {
+            int spins = 0;
+            while (true) {
+              flag_seen = ch_load_flag(pred_flag);
+              if (flag_seen >= kz + 1) break;
+              if (++spins > kChSpinLimit || ((spins & 255) == 0 && ch_load_flag(p.status) != 0)) { give_up(); break; }
+              __builtin_amdgcn_s_sleep(1);
+            }
+          }
+          // (the loads that follow are issued after the count has been seen: the hardware issues this wave's loads in
+          // program order)  The count for the slots to come travels with the partial sums.
+          const int soff = qz0 * (DH * 4);
+          ch_chain_load<0>(cin[0], dqc_voff, dqc_desc, soff); ch_chain_load<32>(cin[1], dqc_voff, dqc_desc, soff);
+          ch_chain_load<64>(cin[2], dqc_voff, dqc_desc, soff); ch_chain_load<96>(cin[3], dqc_voff, dqc_desc, soff);
+          ch_flag_request(flag_v, pred_flag);
         }
         CH_T(3)
-        // ---- dV += P^T dO of block s-1, or dK += dZ^T Q of block s-2; then dQ^T (32 columns x 32 rows) = K^T dZ^T over
-        // the tile's 128 keys.  The operand reads of the second part are issued as the registers of the first fall free,
-        // so that their latency runs under the MFMAs. -----------------------------------------------------------
+        // ---- dV += P^T dO of block s-1, or dK += dZ^T Q of block s-2 -------------------------------------------
         const bool has_w = out ? has_z : (s >= 1 && s - 1 < n);
         const int kw = out ? kz : s - 1;
-        const bool do_dq = has_z && !(kChX & 4);
-        const int z_base = ChLds::kDz + (kz & 1) * ChLds::kStage + rw_off;
-        u32x4 zb[8];
-        f32x16 dq0;
         if (has_w) {
           const int w_base = (out ? ChLds::kDz : ChLds::kP) + (kw & 1) * ChLds::kStage + tr_off;
           const int r_base = (out ? ChLds::kQ + cq_stage * ChLds::kStage : ChLds::kDo + cd_stage * ChLds::kStage) + tr_off + 128 * cp;
+          constexpr int kC1 = 16 * ChLds::kRowBytes;
           u32x2 a_lo[2][4], a_hi[2][4], b_lo[2][2], b_hi[2][2];
           ch_tr_read<0>(a_lo[0][0], a_hi[0][0], w_base); ch_tr_read<64>(a_lo[0][1], a_hi[0][1], w_base);
           ch_tr_read<128>(a_lo[0][2], a_hi[0][2], w_base); ch_tr_read<192>(a_lo[0][3], a_hi[0][3], w_base);
           ch_tr_read<0>(b_lo[0][0], b_hi[0][0], r_base); ch_tr_read<64>(b_lo[0][1], b_hi[0][1], r_base);
-          constexpr int kC1 = 16 * ChLds::kRowBytes;
           ch_tr_read<kC1>(a_lo[1][0], a_hi[1][0], w_base); ch_tr_read<kC1 + 64>(a_lo[1][1], a_hi[1][1], w_base);
           ch_tr_read<kC1 + 128>(a_lo[1][2], a_hi[1][2], w_base); ch_tr_read<kC1 + 192>(a_lo[1][3], a_hi[1][3], w_base);
           ch_tr_read<kC1>(b_lo[1][0], b_hi[1][0], r_base); ch_tr_read<kC1 + 64>(b_lo[1][1], b_hi[1][1], r_base);
@@ -678,59 +670,82 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
 #pragma unroll
             for (int nn = 0; nn < 2; nn++)
               acc[m][nn] = Elem<T>::mfma(as_vec8<T>(ch_join(a_lo[0][m], a_hi[0][m])), as_vec8<T>(ch_join(b_lo[0][nn], b_hi[0][nn])), acc[m][nn]);
-          if (do_dq) {                                       // 12 older reads are still in flight in front of these
-            ch_row_read<0>(zb[0], z_base); ch_row_read<32>(zb[1], z_base); ch_row_read<64>(zb[2], z_base); ch_row_read<96>(zb[3], z_base);
-            ch_landed6<4>(a_lo[1], a_hi[1], b_lo[1], b_hi[1]);
-          } else {
-            ch_landed6<0>(a_lo[1], a_hi[1], b_lo[1], b_hi[1]);
-          }
+          ch_landed6<0>(a_lo[1], a_hi[1], b_lo[1], b_hi[1]);
 #pragma unroll
           for (int m = 0; m < 4; m++)
 #pragma unroll
             for (int nn = 0; nn < 2; nn++)
               acc[m][nn] = Elem<T>::mfma(as_vec8<T>(ch_join(a_lo[1][m], a_hi[1][m])), as_vec8<T>(ch_join(b_lo[1][nn], b_hi[1][nn])), acc[m][nn]);
-        } else if (do_dq) {
-          ch_row_read<0>(zb[0], z_base); ch_row_read<32>(zb[1], z_base); ch_row_read<64>(zb[2], z_base); ch_row_read<96>(zb[3], z_base);
         }
-        if (out == 0 && s >= 1 && s - 1 < n) bump(cd_stage, kChDoStages);
         CH_T(4)
-        if (chain_in && !cdq_loaded) {                       // the count requested at the top of the slot has arrived by now
-          flag_seen = flag_v;
-          if (flag_seen < kz + 1) {
-            int spins = 0;
-            while (true) {
-              flag_seen = ch_load_flag(pred_flag);
-              if (flag_seen >= kz + 1) break;
-              if (++spins > kChSpinLimit || ((spins & 255) == 0 && ch_load_flag(p.status) != 0)) { give_up(); break; }
-              __builtin_amdgcn_s_sleep(1);
-            }
-          }
-          load_chain_in();
+        // ---- everything this wave had in flight has landed by now (the rows requested and the partial dQ stored in the
+        // previous slot, the partial sums just loaded): the previous slot's rows are published, and only then are the
+        // rows three slots ahead requested, so that no wait of this slot is a wait for them ---------------------
+        if (take_in) ch_vm_wait<5>(); else ch_vm_wait<0>();     // all but the five loads of the chain just issued
+        if (pub_flag) {
+          if (lane == 0) __hip_atomic_store(pub_flag, pub_count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          pub_flag = nullptr;
         }
-        // ---- rows three slots ahead, requested AFTER the chain's loads: loads return in order, so a wait for the
-        // partial dQ would otherwise be a wait for these rows as well. ------------------------------------------
+        bool requested = false;
+        // The next tile is claimed late and in three slots: the cursor, then the tile record, then LDS.  (Here, where
+        // nothing is in flight, so that the claim's own memory operations cost the other slots no wait.)
+        if (c == 3) {
+          if (s == f.a) { if (lane == 0) claim_v = atomicAdd(p.head_queue + head, 1); }
+          else if (s == f.a + 1) {
+            claim_v = __builtin_amdgcn_readfirstlane(claim_v);
+            if (claim_v < n_tiles && lane < 6) rec_w = reinterpret_cast<const uint32_t*>(p.k_tiles + claim_v)[lane];
+          } else if (s == f.a + 2) {
+            if (lane < 6) next_lds[lane] = (int)rec_w;
+            if (lane == 0) next_lds[8] = claim_v;
+          }
+        }
+        if (s == f.a + 3) {
+          const int ns = __builtin_amdgcn_readfirstlane(next_lds[8]);
+          have_next = ns < n_tiles;
+          if (have_next) {
+            next_tile.seq_start = __builtin_amdgcn_readfirstlane(next_lds[0]);
+            next_tile.seq_len = __builtin_amdgcn_readfirstlane(next_lds[1]);
+            next_tile.origin = __builtin_amdgcn_readfirstlane(next_lds[2]);
+            next_tile.seq_id = __builtin_amdgcn_readfirstlane(next_lds[3]);
+            const uint32_t lo = __builtin_amdgcn_readfirstlane(next_lds[4]), hi = __builtin_amdgcn_readfirstlane(next_lds[5]);
+            next_tile.carry_base = (int64_t)(((uint64_t)hi << 32) | lo);
+            slot_idx = ns;                                   // used for the flags of the next tile (read at its start)
+          }
+        }
         if (!(kChX & 8)) {
           if (rq_left == 0 && have_next && s + 3 >= S) { request_from(next_tile); }
-          if (rq_left > 0 && (s + 3 < n || s + 3 >= S)) request_rows();
+          if (rq_left > 0 && (s + 3 < n || s + 3 >= S)) { request_rows(); requested = true; }
         }
-        CH_T(2)
+        // ---- dQ^T (32 columns x 32 rows) += K^T dZ^T over the tile's 128 keys ---------------------------------
         if (do_dq) {
+          const int z_base = ChLds::kDz + (kz & 1) * ChLds::kStage + rw_off;
+          u32x4 zb[8];
+          ch_row_read<0>(zb[0], z_base); ch_row_read<32>(zb[1], z_base); ch_row_read<64>(zb[2], z_base); ch_row_read<96>(zb[3], z_base);
           ch_row_read<128>(zb[4], z_base); ch_row_read<160>(zb[5], z_base); ch_row_read<192>(zb[6], z_base); ch_row_read<224>(zb[7], z_base);
+          ch_landed4<4>(zb[0], zb[1], zb[2], zb[3]);
+          f32x16 dq0;
 #pragma unroll
           for (int r = 0; r < 16; r++) dq0[r] = 0.f;
-          ch_landed4<4>(zb[0], zb[1], zb[2], zb[3]);
 #pragma unroll
           for (int kk = 0; kk < 4; kk++) dq0 = Elem<T>::mfma(kstat[kk], as_vec8<T>(zb[kk]), dq0);
           ch_landed4<0>(zb[4], zb[5], zb[6], zb[7]);
 #pragma unroll
           for (int kk = 4; kk < 8; kk++) dq0 = Elem<T>::mfma(kstat[kk], as_vec8<T>(zb[kk]), dq0);
-          // dq0[4a + b]: row qz0 + col, column 32c + 8a + 4*half + b.
-          if (chain_in) {
+          // The partial sums of the tiles below join here.  Younger than their loads are only the row requests (16, when
+          // any) and, in three slots of a tile, a memory operation of the claim (the wait is then stricter than needed).
+          // (Whole-vector bit casts: a bit cast of one element of a vector reads element 0.)
+          if (take_in) {
+            if (requested) ch_vm_wait<16>(); else ch_vm_wait<0>();
+            ch_chain_landed(cin, flag_v);
+            flag_seen = max(flag_seen, __builtin_amdgcn_readfirstlane(flag_v));
 #pragma unroll
-            for (int a4 = 0; a4 < 4; a4++)
+            for (int a4 = 0; a4 < 4; a4++) {
+              const f32x4 v = __builtin_bit_cast(f32x4, cin[a4]);
 #pragma unroll
-              for (int b = 0; b < 4; b++) dq0[4 * a4 + b] += cdq[a4][b];
+              for (int b = 0; b < 4; b++) dq0[4 * a4 + b] += v[b];
+            }
           }
+          // dq0[4a + b]: row qz0 + col, column 32c + 8a + 4*half + b.
           if (final_rows) {
 #pragma unroll
             for (int a4 = 0; a4 < 4; a4++) {
@@ -745,10 +760,12 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
               __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), dqc_rs, dqc_voff + 32 * a4, qz0 * (DH * 4), 0);
             }
           }
+        }
+        if (out == 0 && s >= 1 && s - 1 < n) bump(cd_stage, kChDoStages);
+        if (do_dq) {
           if (!final_rows) { pub_flag = my_flag; pub_count = kz + 1; }
         }
         if (has_z) bump(cq_stage, kChQStages);
-        if (J > 0 && s + 1 < S && !(kChX & 2)) flag_pre = ch_load_flag(pred_flag);      // for the next slot; landed by its top
         CH_T(5)
         lds_barrier();
       }
