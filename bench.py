@@ -111,6 +111,7 @@ class KernelTimer:
         self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
         self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
         self.hip.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
 
     def new_set(self, n=3):
         arr = (ctypes.c_void_p * n)()
@@ -119,6 +120,10 @@ class KernelTimer:
             assert self.hip.hipEventCreate(ctypes.byref(ev)) == 0
             arr[i] = ev
         return arr
+
+    def free(self, arr):
+        for ev in arr:
+            assert self.hip.hipEventDestroy(ctypes.c_void_p(ev)) == 0
 
     def elapsed_ms(self, a, b):
         assert self.hip.hipEventSynchronize(b) == 0
@@ -156,6 +161,8 @@ def time_kernels(inp, native, iters, save_carry=True):
             sums[0] += timer.elapsed_ms(fwd_ev[0], fwd_ev[1])
             sums[1] += timer.elapsed_ms(bwd_ev[0], bwd_ev[1])
             sums[2] += timer.elapsed_ms(bwd_ev[1], bwd_ev[2])
+        timer.free(fwd_ev)
+        timer.free(bwd_ev)
     return [s / iters for s in sums]
 
 
@@ -269,7 +276,14 @@ def main():
     # Algorithmic FLOPs per launch: forward QK^T + PV = 4 D pairs; backward 10 D pairs, of which the dQ kernel is
     # credited with the recompute (QK^T, dO V^T) and dQ = 6 D pairs and the dK/dV kernel with dK, dV = 4 D pairs
     # (its own recompute of QK^T and dO V^T is not algorithmic work).
-    kernels = {"fwd_kernel": (k_fwd, 4 * D * pairs), "bwd_dq_kernel": (k_dq, 6 * D * pairs), "bwd_dkv_kernel": (k_dkv, 4 * D * pairs)}
+    # The chained backward is ONE kernel with all 10 D pairs of the backward and no recompute of its own; what is timed
+    # in front of it is then only the kernel that rebuilds the forward's products, when there is one.
+    if _native.LAST_BWD_KERNELS == 1:
+        kernels = {"fwd_kernel": (k_fwd, 4 * D * pairs), "bwd_chain_kernel": (k_dkv, 10 * D * pairs)}
+        if not save_carry:
+            kernels["fwd_kernel(products only)"] = (k_dq, 2 * D * pairs)
+    else:
+        kernels = {"fwd_kernel": (k_fwd, 4 * D * pairs), "bwd_dq_kernel": (k_dq, 6 * D * pairs), "bwd_dkv_kernel": (k_dkv, 4 * D * pairs)}
     dom = max(kernels, key=lambda n: kernels[n][0])
     dom_ms, dom_flops = kernels[dom]
     achieved = dom_flops / (dom_ms * 1e-3) / 1e12

@@ -133,11 +133,13 @@ typedef struct SbaArgs {
                                   need of a ragged batch; a caller that knows the lengths on the host passes
                                   SbaPlan.carry_slots from sba_plan_host for the exact size.  Must be the same in the
                                   forward, the backward and sba_workspace_bytes. */
-  int32_t backward_kernels;    /* 0 or 1: sba_bwd runs a dQ kernel and a dK/dV kernel.  2: where it applies (head_dim 128,
-                                  16-bit, 16-byte aligned rows, a head count that is a multiple of 8, no add_remainder)
-                                  ONE kernel in which the key tiles of a sequence hand the row prefix sums and the partial
-                                  dQ to each other, the two kernels otherwise.  Must be the same in sba_workspace_bytes
-                                  and sba_bwd. */
+  int32_t backward_kernels;    /* How sba_bwd computes dq, dk, dv.  1: a dQ kernel and a dK/dV kernel.  2: where it applies
+                                  (head_dim 128, 16-bit, 16-byte aligned rows, a head count that is a multiple of 8, no
+                                  add_remainder) ONE kernel in which the key tiles of a sequence hand the row prefix
+                                  sums and the partial dQ to each other through the L2; the two kernels otherwise.
+                                  0: the one kernel where it applies AND is the faster one, which it is while
+                                  max_seqlen * num_heads <= 131072 (measured; in packed mode an overstated max_seqlen
+                                  only costs the faster choice).  Must be the same in sba_workspace_bytes and sba_bwd. */
   int32_t reserved0;
 } SbaArgs;
 
@@ -218,6 +220,14 @@ int sba_fwd_static(const SbaArgs* args);
  * bracket the whole call but only the last group's dQ / dK/dV split.
  */
 int sba_bwd(const SbaArgs* args);
+
+/*
+ * How many attention kernels sba_bwd runs for these arguments on the current device when the workspace holds all
+ * heads: 1 (the chained kernel, see SbaArgs.backward_kernels) or 2 (dQ, then dK/dV); a negative SBA_ERR_* for
+ * arguments sba_bwd would refuse.  Launches nothing.  For callers that attribute the time between trace_events.
+ * No counterpart in the reference (it always runs one kernel with atomics and locks, sb_varlen_bwd.py:541-640).
+ */
+int sba_bwd_kernels(const SbaArgs* args);
 
 #ifdef __cplusplus
 }

@@ -70,7 +70,12 @@ int plan(const SbaArgs* a, Layout* out) {
   L.carry_bytes = align_up((size_t)L.carry_slots_per_head * a->num_heads * sizeof(float), 256);
   size_t chain_bytes = 0;
   L.chain_rows = fixed ? B * T : T;
-  if (a->dtype != SBA_F32 && a->head_dim == 128 && (a->num_heads & 7) == 0 && !a->add_remainder && a->backward_kernels == 2) {
+  // The one-kernel backward is laid out when it is asked for, or (backward_kernels 0) when it is the faster one: it
+  // wins while the longest sequence gives each of a head's workgroups at most four key tiles of 128 (measured on
+  // 256 compute units: beyond that, the partial dQ a tile finds was written too long ago to still be in the L2).
+  const bool chain_shape = a->dtype != SBA_F32 && a->head_dim == 128 && (a->num_heads & 7) == 0 && !a->add_remainder;
+  const bool chain_pays = max_len * a->num_heads <= (int64_t)512 * 256;
+  if (chain_shape && (a->backward_kernels == 2 || (a->backward_kernels == 0 && chain_pays))) {
     size_t c = off;
     L.off_chain_zero = c;
     L.off_chain_c = c;      c = align_up(c + (size_t)a->num_heads * L.chain_rows * 8, 256);
@@ -291,6 +296,27 @@ int sba_fwd_static(const SbaArgs* a) {
 
 namespace {
 
+// Whether every tensor of the backward allows 16-byte accesses.
+bool bwd_vec_ok(const SbaArgs* a) {
+  const bool fixed = a->cu_seqlens == nullptr;
+  const size_t es = elem_size(a->dtype);
+  const int64_t max_rows = (a->max_seqlen > 0 && a->max_seqlen < a->total_tokens) ? a->max_seqlen : a->total_tokens;
+  bool v16 = (a->head_dim % (16 / (int)es)) == 0;
+  for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
+    if (t->ptr) v16 = v16 && vec16(*t, es, fixed, max_rows);
+  return v16;
+}
+// Whether one pass over the heads `a` describes runs the one-kernel backward (its buffers are laid out and the
+// tensors and the device allow it).
+bool bwd_is_chained(const SbaArgs* a, const Layout& L) {
+  sba::BwdParams p{};
+  p.vec_ok = bwd_vec_ok(a) ? 1 : 0;
+  p.head_dim = a->head_dim;
+  p.num_heads = a->num_heads;
+  p.add_rem = a->add_remainder ? 1 : 0;
+  return a->dtype != SBA_F32 && L.chain_zero_bytes > 0 && sba::chain_supported(p);
+}
+
 // One pass of the backward over the heads `a` describes (all of them, or one group of a larger call: `stat_heads` is
 // the head count of the caller's row_stat array, `first`/`last` say which trace events this pass records).
 int bwd_pass(const SbaArgs* a, int64_t stat_heads, bool first, bool last) {
@@ -338,13 +364,9 @@ int bwd_pass(const SbaArgs* a, int64_t stat_heads, bool first, bool last) {
   p.head_queue = (int32_t*)(ws + L.off_queue);
   p.max_tiles = (int32_t)L.max_q_tiles;
   p.total_tokens = a->total_tokens;
-  const int64_t max_rows = (a->max_seqlen > 0 && a->max_seqlen < a->total_tokens) ? a->max_seqlen : a->total_tokens;
-  bool v16 = (a->head_dim % (16 / (int)es)) == 0;
-  for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
-    if (t->ptr) v16 = v16 && vec16(*t, es, fixed, max_rows);
-  p.vec_ok = v16 ? 1 : 0;
+  p.vec_ok = bwd_vec_ok(a) ? 1 : 0;
   // One kernel (the key tiles of a sequence hand C and partial dQ to each other) where it applies, else dQ then dK/dV.
-  const bool chain = a->dtype != SBA_F32 && L.chain_zero_bytes > 0 && sba::chain_supported(p);
+  const bool chain = bwd_is_chained(a, L);
   if (chain) {
     p.chain_c = (uint32_t*)(ws + L.off_chain_c);
     p.chain_flags = (int32_t*)(ws + L.off_chain_flags);
@@ -381,6 +403,7 @@ int bwd_pass(const SbaArgs* a, int64_t stat_heads, bool first, bool last) {
     f.attend_current = p.attend_current;
     f.max_tiles = (int32_t)L.max_q_tiles;
     f.total_tokens = a->total_tokens;
+    const int64_t max_rows = (a->max_seqlen > 0 && a->max_seqlen < a->total_tokens) ? a->max_seqlen : a->total_tokens;
     bool fv16 = (a->head_dim % (16 / (int)es)) == 0;
     for (const SbaTensor* t : {&a->q, &a->k}) fv16 = fv16 && vec16(*t, es, fixed, max_rows);
     f.vec_ok = fv16 ? 1 : 0;
@@ -403,6 +426,14 @@ int bwd_pass(const SbaArgs* a, int64_t stat_heads, bool first, bool last) {
 }  // namespace
 
 extern "C" {
+
+int sba_bwd_kernels(const SbaArgs* a) {
+  if (!a) return SBA_ERR_NULL;
+  Layout L;
+  const int st = plan(a, &L);
+  if (st != SBA_OK) return st;
+  return bwd_is_chained(a, L) ? 1 : 2;
+}
 
 int sba_bwd(const SbaArgs* a) {
   if (!a) return SBA_ERR_NULL;

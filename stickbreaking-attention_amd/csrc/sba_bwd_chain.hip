@@ -171,7 +171,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
   constexpr int kRowStride = lds_stride<DH>();           // elements; P / dZ tiles use the same stride
   constexpr int kSteps = DH / 16;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  T* lds = reinterpret_cast<T*>(lds_raw);
   typedef __attribute__((address_space(3))) unsigned char lds_u8;
   typedef __attribute__((address_space(3))) void lds_void;
 
@@ -505,15 +504,16 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
     vec8 kstat[kSteps];                                      // K^T of the tile for columns 32c..: A operand of dQ^T = K^T dZ^T
     int cq_stage = 0, cd_stage = 0;                          // stages of the blocks to contract (Q: 2 behind, dO: 1 behind)
     auto bump = [](int& st, int n_st) { st = st == n_st - 1 ? 0 : st + 1; };
-    // Row requests.  This wave brings in rows 8c .. 8c+7 of a block: one 4-byte-per-lane direct-to-LDS load per row (a
-    // row of 128 16-bit elements is exactly 64 lanes x 4 bytes, so the padded row layout stays; no staging registers,
-    // no LDS write instructions).  The requests run three slots ahead of the math, beyond the end of the tile the
+    // Row requests.  This wave brings in rows 8c .. 8c+7 of a block with direct-to-LDS loads of 16 bytes per lane (no
+    // staging registers, no LDS write instructions).  Such a load writes the lanes' 16-byte pieces back to back, and
+    // the rows are padded in LDS (19 pieces of which 16 hold data), so the lanes are laid over the padded rows: lane
+    // i of load k covers piece 64k + i of the wave's 152; a lane over padding asks for an address outside the
+    // buffer and leaves zeros there.  The requests run three slots ahead of the math, beyond the end of the tile the
     // wave contracts, so they keep their own descriptors: the rows of the sequence being requested from, the next
     // block, and how many blocks of that tile are left.
     __amdgpu_buffer_rsrc_t rq_q, rq_do;
     int rq_qsb = 0, rq_dosb = 0, rq_block = 0, rq_left = 0;
     int rq_qst = 0, rq_dst = 0;                              // stages of the next row block to request
-    const int rq_voff = lane * 4;
     auto request_from = [&](const Tile& tl) {
       const Facts ft = facts_of(tl);
       const T* qb = (const T*)p.q.ptr + tl.seq_id * p.q.sb + head * p.q.sh + (int64_t)tl.seq_start * p.q.st;
@@ -525,12 +525,18 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
     auto request_rows = [&]() {
       lds_u8* qd = (lds_u8*)lds_raw + ChLds::kQ + rq_qst * ChLds::kStage + 8 * c * ChLds::kRowBytes;
       lds_u8* dd = (lds_u8*)lds_raw + ChLds::kDo + rq_dst * ChLds::kStage + 8 * c * ChLds::kRowBytes;
-      int qo = (kChRows * rq_block + 8 * c) * rq_qsb, dob_ = (kChRows * rq_block + 8 * c) * rq_dosb;
+      const int qo = (kChRows * rq_block + 8 * c) * rq_qsb, dob_ = (kChRows * rq_block + 8 * c) * rq_dosb;
+      constexpr int kPieces = 8 * ChLds::kRowBytes / 16;     // 152
+      constexpr int kOutside = 0x7ffffff0;                   // past every buffer: reads as zero
 #pragma unroll
-      for (int i = 0; i < 8; i++) {                           // rows beyond the sequence read as zero
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rq_q, (lds_void*)(qd + i * ChLds::kRowBytes), 4, rq_voff, qo, 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rq_do, (lds_void*)(dd + i * ChLds::kRowBytes), 4, rq_voff, dob_, 0, 0);
-        qo += rq_qsb; dob_ += rq_dosb;
+      for (int k = 0; k < 3; k++) {                          // rows beyond the sequence read as zero
+        const int piece = 64 * k + lane;
+        const int row = (piece * 27) >> 9, cc = piece - 19 * row;           // piece / 19 for piece < 152
+        const int vq = cc < 16 ? row * rq_qsb + 16 * cc : kOutside, vd = cc < 16 ? row * rq_dosb + 16 * cc : kOutside;
+        if (64 * k + 64 <= kPieces || piece < kPieces) {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rq_q, (lds_void*)(qd + 1024 * k), 16, vq, qo, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rq_do, (lds_void*)(dd + 1024 * k), 16, vd, dob_, 0, 0);
+        }
       }
       bump(rq_qst, kChQStages); bump(rq_dst, kChDoStages);
       --rq_block; --rq_left;
@@ -571,6 +577,8 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
       const Facts f = facts_of(tile);
       const int L = f.L, J = f.J, n = f.n, S = f.S;
       bool have_next = false;
+      bool rq_next = false;                                  // the requests have moved on to the next tile (a tile of one or
+                                                             // two row blocks is fully requested before this one ends)
       int32_t* const my_flag = p.chain_flags + ((int64_t)head * p.chain_tile_cap + slot_idx) * 8 + c;
       const int32_t* const pred_flag = my_flag - 8;
       int flag_seen = 0;                                     // the tile below's count for this wave's columns, as last read
@@ -586,7 +594,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
       for (int s = 0; s < S; ++s) {
         // ---- top of the slot: everything this wave has in flight completes, then it is published ---------------
         CH_T(6)
-        CH_T(0)
         if (s == 0) {
           // K^T of this tile for the dQ contraction, through the wave's scratch: [32 keys][32 columns] at a time,
           // gathered down the keys by the transpose read.  The previous tile's results leave first (same scratch).
@@ -682,6 +689,7 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
         // previous slot, the partial sums just loaded): the previous slot's rows are published, and only then are the
         // rows three slots ahead requested, so that no wait of this slot is a wait for them ---------------------
         if (take_in) ch_vm_wait<5>(); else ch_vm_wait<0>();     // all but the five loads of the chain just issued
+        CH_T(0)
         if (pub_flag) {
           if (lane == 0) __hip_atomic_store(pub_flag, pub_count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           pub_flag = nullptr;
@@ -713,9 +721,10 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
           }
         }
         if (!(kChX & 8)) {
-          if (rq_left == 0 && have_next && s + 3 >= S) { request_from(next_tile); }
+          if (!rq_next && rq_left == 0 && have_next && s + 3 >= S) { request_from(next_tile); rq_next = true; }
           if (rq_left > 0 && (s + 3 < n || s + 3 >= S)) { request_rows(); requested = true; }
         }
+        CH_T(2)
         // ---- dQ^T (32 columns x 32 rows) += K^T dZ^T over the tile's 128 keys ---------------------------------
         if (do_dq) {
           const int z_base = ChLds::kDz + (kz & 1) * ChLds::kStage + rw_off;
@@ -731,12 +740,13 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
           ch_landed4<0>(zb[4], zb[5], zb[6], zb[7]);
 #pragma unroll
           for (int kk = 4; kk < 8; kk++) dq0 = Elem<T>::mfma(kstat[kk], as_vec8<T>(zb[kk]), dq0);
-          // The partial sums of the tiles below join here.  Younger than their loads are only the row requests (16, when
+          // The partial sums of the tiles below join here.  Younger than their loads are only the row requests (6, when
           // any) and, in three slots of a tile, a memory operation of the claim (the wait is then stricter than needed).
           // (Whole-vector bit casts: a bit cast of one element of a vector reads element 0.)
           if (take_in) {
-            if (requested) ch_vm_wait<16>(); else ch_vm_wait<0>();
+            if (requested) ch_vm_wait<6>(); else ch_vm_wait<0>();
             ch_chain_landed(cin, flag_v);
+            CH_T(7)
             flag_seen = max(flag_seen, __builtin_amdgcn_readfirstlane(flag_v));
 #pragma unroll
             for (int a4 = 0; a4 < 4; a4++) {

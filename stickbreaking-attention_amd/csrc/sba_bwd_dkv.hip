@@ -281,7 +281,7 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
   for (int slot = w; slot < n_tiles;) {
   const Tile tile = next_tile;
   if (threadIdx.x == 0) *next_slot_lds = wph + atomicAdd(p.head_queue + head, 1);
-  const int L = tile.seq_len, j0 = tile.origin, ac = p.attend_current, D = DH;
+  const int L = tile.seq_len, j0 = tile.origin, ac = p.attend_current;
   const int64_t tok0 = tile.seq_start;
   const int jt = j0 / kBlockK;
 
@@ -292,10 +292,10 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
 
     const int rg = wave >> 1, group = wave & 1;
     const int jb = j0 + 32 * group;          // first key of this wave's sub-tile
-    const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
-    const T* kb = (const T*)p.k.ptr + tile.seq_id * p.k.sb + head * p.k.sh + tok0 * p.k.st;
-    const T* vb = (const T*)p.v.ptr + tile.seq_id * p.v.sb + head * p.v.sh + tok0 * p.v.st;
-    const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
+    [[maybe_unused]] const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
+    [[maybe_unused]] const T* kb = (const T*)p.k.ptr + tile.seq_id * p.k.sb + head * p.k.sh + tok0 * p.k.st;
+    [[maybe_unused]] const T* vb = (const T*)p.v.ptr + tile.seq_id * p.v.sb + head * p.v.sh + tok0 * p.v.st;
+    [[maybe_unused]] const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
     const int64_t slot0 = (int64_t)head * p.carry_head_stride + tile.carry_base +
                           carry_offset(2 * jt + group, n_qt) - (int64_t)kBlockQ * (jt >> 1);      // + row
     const float* carry = p.carry + slot0;
@@ -435,8 +435,8 @@ __global__ __launch_bounds__(kDkv3Threads) void bwd_dkv3_kernel(BwdParams p) {
     // The consumers also move the query tiles global -> registers -> LDS (they have the issue slots to spare):
     // tile t+1 is written at the top of step t from registers loaded during step t-1, then tile t+2 is requested;
     // the barrier that ends a step is the only point that waits for those loads.
-    const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
-    const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
+    [[maybe_unused]] const T* qb = (const T*)p.q.ptr + tile.seq_id * p.q.sb + head * p.q.sh + tok0 * p.q.st;
+    [[maybe_unused]] const T* dob = (const T*)p.d_o.ptr + tile.seq_id * p.d_o.sb + head * p.d_o.sh + tok0 * p.d_o.st;
     const RowSource<T> qsrc = make_row_source<T, true>(qb, p.q.st, L, D), dosrc = make_row_source<T, true>(dob, p.d_o.st, L, D);
     if (n_steps > 0) {                                       // rows of step 0 were requested a tile ago
       cq.store(lds + Lds::kQ);

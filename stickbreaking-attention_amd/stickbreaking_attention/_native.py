@@ -55,7 +55,7 @@ class SbaPlan(ctypes.Structure):
                 ("pairs", ctypes.c_int64)]
 
 
-EXPORTS = ("sba_version", "sba_strerror", "sba_workspace_bytes", "sba_plan_host", "sba_fwd", "sba_fwd_static", "sba_bwd")
+EXPORTS = ("sba_version", "sba_strerror", "sba_workspace_bytes", "sba_plan_host", "sba_fwd", "sba_fwd_static", "sba_bwd", "sba_bwd_kernels")
 STATUS_OFFSET = 8        # SBA_STATUS_OFFSET: the scheduler's status word inside the workspace
 # Debugging aid for the tests: fill the carry buffer and the workspaces with NaN bit patterns before every launch,
 # so that a kernel reading a slot nobody wrote shows up as NaN instead of passing on whatever the allocator returned.
@@ -64,8 +64,10 @@ POISON = os.environ.get("SBA_DEBUG_POISON", "0") == "1"
 # and raise on a schedule the device refused.  Without it a bad ``cu_seqlens`` that only exists on the device yields
 # all-zero outputs and gradients and no error.
 DEBUG_CHECK = os.environ.get("SBA_DEBUG_CHECK", "0") == "1"
-# SbaArgs.backward_kernels: 0 / 1 = dQ then dK/dV, 2 = one chained kernel where it applies.
+# SbaArgs.backward_kernels: 0 = the library chooses, 1 = dQ then dK/dV, 2 = one chained kernel where it applies.
 BACKWARD_KERNELS = int(os.environ.get("SBA_BACKWARD_KERNELS", "0"))
+# Attention kernels the last traced backward ran: 1 (chained) or 2 (set when TRACE_EVENTS is).
+LAST_BWD_KERNELS = 0
 _STATUS_TEXT = {1: "cu_seqlens is not a non-decreasing sequence within [0, total_tokens] (or its leading entry is not 0)",
                 2: "the carry buffer is too small for these sequence lengths (max_seqlens understated?)",
                 3: "one-kernel backward: a workgroup gave up waiting for the key tile below its own",
@@ -99,7 +101,7 @@ def lib():
         handle.sba_workspace_bytes.argtypes = [ctypes.POINTER(SbaArgs)] + [ctypes.POINTER(ctypes.c_size_t)] * 3
         handle.sba_plan_host.restype = ctypes.c_int
         handle.sba_plan_host.argtypes = [ctypes.POINTER(SbaArgs), ctypes.c_void_p, ctypes.POINTER(SbaPlan)]
-        for name in ("sba_fwd", "sba_fwd_static", "sba_bwd"):
+        for name in ("sba_fwd", "sba_fwd_static", "sba_bwd", "sba_bwd_kernels"):
             fn = getattr(handle, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.POINTER(SbaArgs)]
@@ -286,6 +288,9 @@ def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leadin
         a.workspace, a.workspace_bytes = ws.data_ptr(), nbytes
         if POISON:
             _poison(ws)
+        if TRACE_EVENTS is not None:
+            global LAST_BWD_KERNELS
+            LAST_BWD_KERNELS = lib().sba_bwd_kernels(ctypes.byref(a))
         _check(lib().sba_bwd(ctypes.byref(a)), "sba_bwd")
         if DEBUG_CHECK:
             check_status(ws, "sba_bwd")

@@ -30,7 +30,7 @@ def declared_functions():
 def test_library_exports_every_declared_symbol(native):
     names = declared_functions()
     assert set(names) == set(native.EXPORTS) == {"sba_version", "sba_strerror", "sba_workspace_bytes", "sba_plan_host", "sba_fwd",
-                                                 "sba_fwd_static", "sba_bwd"}
+                                                 "sba_fwd_static", "sba_bwd", "sba_bwd_kernels"}
     lib = native.lib()
     for n in names:
         assert hasattr(lib, n), n

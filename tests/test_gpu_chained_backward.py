@@ -1,0 +1,132 @@
+"""GPU tests of the one-kernel ("chained") backward: `SbaArgs.backward_kernels = 2`, reached through the Python
+operators and the C ABI.
+
+The chained kernel must give what the two-kernel backward gives up to the rounding of a different summation order
+(dq is summed over key tiles in fp32 in both, but the chained kernel carries the partial sums through memory), and
+both must meet the oracle to the bar of test_gpu_parity.py: max-abs error <= 2e-2, or one ulp of the 16-bit output
+type where |reference| is large.  The status word of the workspace is read back after every launch (a wait that
+ran out, or workgroups of a head on different XCDs, would show there and raise).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import sb_oracle as orc
+from test_gpu_parity import error_bound, small_case, tol_check
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def native_checked():
+    from stickbreaking_attention import _native
+
+    saved = (_native.DEBUG_CHECK, _native.BACKWARD_KERNELS)
+    _native.DEBUG_CHECK = True
+    yield _native
+    _native.DEBUG_CHECK, _native.BACKWARD_KERNELS = saved
+
+
+def grads_varlen(native, mode, dev_t, cu, lengths, attend_current):
+    from stickbreaking_attention import sb_attn_varlen
+
+    native.BACKWARD_KERNELS = mode
+    q, k, v, do, drem = dev_t
+    q, k, v = (t.detach().clone().requires_grad_() for t in (q, k, v))
+    o, rem = sb_attn_varlen(q, k, v, cu.to(q.device), max(lengths), zero_start=False, attend_current=attend_current)
+    g = torch.autograd.grad([o, rem], [q, k, v], [do, drem])
+    torch.cuda.synchronize()
+    return [t.detach() for t in g]
+
+
+CASES = [
+    # label, H, lengths
+    ("one-row", 8, [1]),
+    ("one-block", 8, [32]),
+    ("block-plus-one", 8, [33]),
+    ("one-tile", 8, [128]),
+    ("tile-plus-one", 8, [129]),
+    ("ragged", 8, [200, 1, 77, 130]),
+    ("two-chains", 8, [1000, 333]),
+    ("sixteen-tiles", 8, [2048]),
+    ("many-heads", 32, [700, 64, 300]),
+    ("long-and-short", 16, [4096, 64, 700]),
+    # more key tiles than workgroups of a head, among them tiles of one or two row blocks taken as a workgroup's
+    # second or later tile
+    ("several-tiles-per-workgroup", 32, [300] * 12),
+    ("short-last-tiles", 32, [290, 130, 161, 257, 420, 129, 385, 33, 1, 513, 140, 260, 200, 100, 390]),
+]
+
+
+@pytest.mark.parametrize("label,H,lengths", CASES, ids=[c[0] for c in CASES])
+@pytest.mark.parametrize("attend_current", [False, True], ids=["strict", "attend-current"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_chained_backward_matches_oracle_and_two_kernels(gpu_device, native_checked, label, H, lengths, attend_current, dtype):
+    if dtype == torch.float16 and sum(lengths) > 1500:
+        pytest.skip("fp16 is covered on the short cases")
+    host, dev_t, cu = small_case(H, 128, lengths, dtype, seed=len(lengths) + H)
+    two = grads_varlen(native_checked, 1, dev_t, cu, lengths, attend_current)
+    one = grads_varlen(native_checked, 2, dev_t, cu, lengths, attend_current)
+    again = grads_varlen(native_checked, 2, dev_t, cu, lengths, attend_current)
+    q, k, v, do, drem = host
+    ref = orc.varlen_stream(q, k, v, cu, do=do, drem=drem, dtype=torch.float64, attend_current=attend_current)
+    for name, a, b, c, r in zip(("dq", "dk", "dv"), one, two, again, ref[2:]):
+        tol_check(name, a, r, dtype, f"chained {label}")
+        # no atomics anywhere: a second run gives the same bits
+        assert torch.equal(a, c), f"{label}: {name} differs between two runs of the chained kernel"
+        # against the two-kernel backward: both within the bound of the oracle, so within twice the bound of each other
+        diff = (a.double().cpu() - b.double().cpu()).abs()
+        assert (diff <= 2 * error_bound(r.double(), dtype)).all(), f"{label}: {name} chained vs two kernels {diff.max().item():.3e}"
+
+
+def test_chained_backward_fixed_length(gpu_device, native_checked):
+    """`sb_attn` (batch, head, token, head_dim): the chain buffers are addressed per batch element."""
+    from stickbreaking_attention import sb_attn
+
+    B, H, L, D = 3, 8, 300, 128
+    g = torch.Generator().manual_seed(5)
+    q, k, v, do = (torch.randn(B, H, L, D, generator=g).bfloat16() for _ in range(4))
+    drem = torch.randn(B, H, L, generator=g).bfloat16()
+    out = {}
+    for mode in (1, 2):
+        native_checked.BACKWARD_KERNELS = mode
+        qd, kd, vd = (t.to(gpu_device).requires_grad_() for t in (q, k, v))
+        o, rem = sb_attn(qd, kd, vd)
+        out[mode] = torch.autograd.grad([o, rem], [qd, kd, vd], [do.to(gpu_device), drem.to(gpu_device)])
+        torch.cuda.synchronize()
+    for b in range(B):
+        cu = torch.tensor([L], dtype=torch.int32)
+        ref = orc.varlen_stream(q[b], k[b], v[b], cu, do=do[b], drem=drem[b], dtype=torch.float64)
+        for name, a, r in zip(("dq", "dk", "dv"), out[2], ref[2:]):
+            tol_check(name, a[b], r, torch.bfloat16, f"chained fixed-length batch {b}")
+
+
+def _bwd_kernels(native, q, lengths, backward_kernels, add_remainder=False, max_seqlen=None):
+    """`sba_bwd_kernels` for a packed call on tensors shaped like `q` (nothing is launched)."""
+    cu = torch.tensor(np.cumsum(lengths), dtype=torch.int32, device=q.device)
+    native.BACKWARD_KERNELS = backward_kernels
+    a = native._base_args(q, cu, False, max_seqlen or max(lengths), 1.0, False)
+    a.add_remainder = 1 if add_remainder else 0
+    for f in ("q", "k", "v", "d_o", "dq", "dk", "dv"):
+        setattr(a, f, native._tensor(q, False))
+    return native.lib().sba_bwd_kernels(ctypes.byref(a))
+
+
+def test_which_backward_runs(gpu_device, native_checked):
+    """The one-kernel backward runs only where it applies; left to the library (0) only where it is the faster one."""
+    n = native_checked
+    q = torch.zeros(8, 1024, 128, dtype=torch.bfloat16, device=gpu_device)
+    assert _bwd_kernels(n, q, [1024], 2) == 1
+    assert _bwd_kernels(n, q, [1024], 1) == 2
+    assert _bwd_kernels(n, q, [1024], 0) == 1
+    assert _bwd_kernels(n, q, [1024], 2, add_remainder=True) == 2
+    assert _bwd_kernels(n, q[:7], [1024], 2) == 2                                    # 7 heads
+    assert _bwd_kernels(n, q[..., :64], [1024], 2) == 2                              # head_dim 64 (and unaligned rows)
+    assert _bwd_kernels(n, q.float(), [1024], 2) == 2                                # fp32
+    big = torch.zeros(32, 8192, 128, dtype=torch.bfloat16, device=gpu_device)
+    assert _bwd_kernels(n, big, [8192], 0) == 2                                      # 8192 * 32 > 131072
+    assert _bwd_kernels(n, big, [4096, 4096], 0) == 1
+    assert _bwd_kernels(n, big, [4096, 4096], 0, max_seqlen=8192) == 2               # an overstated bound decides
+    assert _bwd_kernels(n, big, [8192], 2) == 1
