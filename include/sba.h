@@ -101,7 +101,11 @@ typedef struct SbaArgs {
   SbaTensor q, k, v;           /* inputs */
   SbaTensor o;                 /* forward output, dtype of q */
   SbaVector rem;               /* forward output, dtype of q: 1 - sum_j A_ij */
-  float* row_stat;             /* forward output, fp32, contiguous (H, T) / (B, H, L): log2(rem) */
+  float* row_stat;             /* forward output, fp32, contiguous (H, T) / (B, H, L): log2(rem).  -inf (never NaN) for a
+                                  row whose remainder underflows fp32 -- a few hundred saturated keys do that -- where
+                                  the reference keeps a finite neg_log_acc (sb_varlen_fwd.py:156-181); rem is 0 or denormal in both,
+                                  and the backward here does not read row_stat except with add_remainder, where only
+                                  exp2(row_stat) = rem enters. */
   float* carry;                /* forward output (optional, NULL when no backward will follow) and backward input:
                                   for every row and every 32-key sub-tile the row sweeps, the product of (1 - sigma)
                                   over the keys between that sub-tile and the row.  sba_workspace_bytes sizes it. */
@@ -127,12 +131,15 @@ typedef struct SbaArgs {
                                   kernel stripped of everything else: the state kept between the passes is then O(tokens)
                                   as in the reference (q, k, v and, with add_remainder, row_stat), at the price of one more
                                   kernel in the backward.  Must be the same in sba_workspace_bytes and sba_bwd.  16-bit
-                                  dtypes only. */
+                                  dtypes only.  In sba_fwd (with carry = NULL) it makes the forward's scheduler check the
+                                  carry capacity exactly as the backward's will, so that an understated max_seqlen or
+                                  carry_slots voids both passes and not the backward alone. */
   int64_t carry_slots;         /* fp32 slots of `carry` (and of the backward's prefix plane) per head.  0: sized from
                                   the bound total_tokens * max_seqlen / 64 (packed mode), which is several times the
                                   need of a ragged batch; a caller that knows the lengths on the host passes
                                   SbaPlan.carry_slots from sba_plan_host for the exact size.  Must be the same in the
-                                  forward, the backward and sba_workspace_bytes. */
+                                  forward, the backward and sba_workspace_bytes.  Ignored in fixed-length mode, whose
+                                  exact count follows from the shape. */
   int32_t backward_kernels;    /* How sba_bwd computes dq, dk, dv.  1: a dQ kernel and a dK/dV kernel.  2: where it applies
                                   (head_dim 128, 16-bit, 16-byte aligned rows, a head count that is a multiple of 8, no
                                   add_remainder) ONE kernel in which the key tiles of a sequence hand the row prefix

@@ -60,7 +60,8 @@ int plan(const SbaArgs* a, Layout* out) {
     L.carry_slots_per_head = cdiv(T * max_len, 64) + 6 * T + 512 * B;
   }
   // A caller that knows the lengths passes the exact count (sba_plan_host); the scheduler checks it on the device.
-  if (a->carry_slots > 0) L.carry_slots_per_head = a->carry_slots;
+  // (Fixed-length mode knows its exact count above; a caller's figure is not needed there and is ignored.)
+  if (a->carry_slots > 0 && !fixed) L.carry_slots_per_head = a->carry_slots;
   size_t off = 0;
   L.off_counts = off;      off = align_up(off + 256, 256);
   L.off_q_tiles = off;     off = align_up(off + (size_t)L.max_q_tiles * sizeof(sba::Tile), 256);
@@ -242,7 +243,9 @@ int fwd_on(const SbaArgs* a, char* ws, size_t ws_bytes, bool ws_is_static) {
   if (ws_is_static && ws_bytes < L.fwd_bytes) return SBA_ERR_TOO_LARGE;
   if (!ws || ((uintptr_t)ws & 255) || ws_bytes < L.fwd_bytes) return SBA_ERR_WORKSPACE;
   hipStream_t stream = (hipStream_t)a->stream;
-  if ((st = run_sched(a, ws, L, false, a->carry != nullptr, kBlockK, stream)) != SBA_OK) return st;
+  // The carry offsets are laid out (and the capacity checked) when products are recorded, and also when the backward
+  // will rebuild them: both passes then agree on whether the schedule stands.
+  if ((st = run_sched(a, ws, L, false, a->carry != nullptr || a->recompute_carry, kBlockK, stream)) != SBA_OK) return st;
 
   sba::FwdParams p{};
   p.q = ref(a->q, fixed); p.k = ref(a->k, fixed); p.v = ref(a->v, fixed); p.o = ref(a->o, fixed);

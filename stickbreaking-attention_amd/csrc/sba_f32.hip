@@ -13,6 +13,7 @@
 //             LDS; dk/dv are flushed once per step with fp32 atomics (and zero-filled by a fill kernel first).
 //             Summation order across workgroups is therefore not fixed; differences are at the 1e-7 level.
 #include "sba_device.hpp"
+#include "sba_host.hpp"
 #include "sba_params.hpp"
 
 namespace sba {
@@ -259,9 +260,11 @@ hipError_t launch_bwd_f32(const BwdParams& p, int batches, int64_t tokens, int m
   // dq is stored, not accumulated, but only for rows that belong to a sequence: the fill covers the others.
   hipLaunchKernelGGL(fill_zero_rows_kernel, dim3(1024), dim3(256), 0, stream, p.dq, batches, p.num_heads, tokens, p.head_dim);
   if (hipGetLastError() != hipSuccess) return hipErrorLaunchFailure;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_f32_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(BwdF32Lds));
+  static std::atomic<uint64_t> lds_done{0};
+  int dev = 0, cus = 0;
+  hipError_t e = device_cus(&dev, &cus);
   if (e != hipSuccess) return e;
+  if ((e = raise_lds_limit(&bwd_f32_kernel, lds_done, dev, sizeof(BwdF32Lds))) != hipSuccess) return e;
   hipLaunchKernelGGL(bwd_f32_kernel, dim3((unsigned)(max_q_tiles * p.num_heads * kF32Split)), dim3(kThreads), sizeof(BwdF32Lds), stream, p);
   return hipGetLastError();
 }

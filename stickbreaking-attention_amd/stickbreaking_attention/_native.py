@@ -236,6 +236,23 @@ def _poison(t: torch.Tensor):
     t.view(torch.uint8).fill_(0xFF)          # every fp32 / 16-bit word becomes a NaN pattern, every int32 becomes -1
 
 
+# Workspace sizes depend on the shape and the flags of a call only (never on pointers or on the lengths behind
+# cu_seqlens), so they are asked for once per distinct call and remembered.
+_WS_BYTES = {}
+
+
+def _workspace_bytes(a: SbaArgs):
+    """(forward workspace, backward workspace, carry) sizes in bytes for these arguments."""
+    key = (a.dtype, a.num_heads, a.head_dim, a.num_seqs, a.total_tokens, a.max_seqlen, bool(a.cu_seqlens), a.cu_is_int64,
+           a.cu_has_leading_zero, a.attend_current, a.add_remainder, a.recompute_carry, a.carry_slots, a.backward_kernels)
+    got = _WS_BYTES.get(key)
+    if got is None:
+        f, b, c = ctypes.c_size_t(0), ctypes.c_size_t(0), ctypes.c_size_t(0)
+        _check(lib().sba_workspace_bytes(ctypes.byref(a), ctypes.byref(f), ctypes.byref(b), ctypes.byref(c)), "sba_workspace_bytes")
+        got = _WS_BYTES[key] = (f.value, b.value, c.value)
+    return got
+
+
 def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, carry_slots, logit_scale, attend_current, add_remainder,
                 o, rem, neg_log_acc, carry):
     fixed = cu_seqlens is None
@@ -245,17 +262,20 @@ def _launch_fwd(q, k, v, cu_seqlens, cu_has_leading_zero, max_seqlen, carry_slot
         a.q, a.k, a.v, a.o = (_tensor(t, fixed) for t in (q, k, v, o))
         a.rem = _vector(rem, fixed)
         a.row_stat = neg_log_acc.data_ptr()
-        need, need_carry = ctypes.c_size_t(0), ctypes.c_size_t(0)
-        _check(lib().sba_workspace_bytes(ctypes.byref(a), ctypes.byref(need), None, ctypes.byref(need_carry)), "sba_workspace_bytes")
-        ws = torch.empty(need.value, dtype=torch.uint8, device=q.device)
-        a.workspace, a.workspace_bytes = ws.data_ptr(), need.value
+        if carry.numel() == 0 and q.dtype != torch.float32:
+            # no products kept: a backward, if one follows, rebuilds them, and the forward's scheduler checks their
+            # capacity as that backward's will (both passes void, or neither)
+            a.recompute_carry = 1
+        need_fwd, _, need_carry_bytes = _workspace_bytes(a)
+        ws = torch.empty(need_fwd, dtype=torch.uint8, device=q.device)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), need_fwd
         if POISON:
             _poison(ws)
             if carry.numel() > 0:
                 _poison(carry)
         if carry.numel() > 0:
-            if carry.numel() * 4 < need_carry.value:
-                raise RuntimeError(f"carry buffer too small: {carry.numel() * 4} < {need_carry.value} bytes")
+            if carry.numel() * 4 < need_carry_bytes:
+                raise RuntimeError(f"carry buffer too small: {carry.numel() * 4} < {need_carry_bytes} bytes")
             a.carry = carry.data_ptr()
         _check(lib().sba_fwd(ctypes.byref(a)), "sba_fwd")
         if DEBUG_CHECK:
@@ -275,15 +295,13 @@ def _launch_bwd(do, drem, q, k, v, carry, neg_log_acc, cu_seqlens, cu_has_leadin
             a.carry = carry.data_ptr()
         else:
             a.recompute_carry = 1        # the forward kept no products: rebuild them in the backward's workspace
-        need = ctypes.c_size_t(0)
-        _check(lib().sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(need), None), "sba_workspace_bytes")
-        nbytes = need.value
+        nbytes = _workspace_bytes(a)[1]
         if BWD_WORKSPACE_LIMIT is not None and nbytes > BWD_WORKSPACE_LIMIT:
             # the smallest workspace the library accepts is the one of a single head
             heads, a.num_heads = a.num_heads, 1
-            _check(lib().sba_workspace_bytes(ctypes.byref(a), None, ctypes.byref(need), None), "sba_workspace_bytes")
+            one_head = _workspace_bytes(a)[1]
             a.num_heads = heads
-            nbytes = max(BWD_WORKSPACE_LIMIT, need.value)
+            nbytes = max(BWD_WORKSPACE_LIMIT, one_head)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
         a.workspace, a.workspace_bytes = ws.data_ptr(), nbytes
         if POISON:

@@ -48,7 +48,15 @@ def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, zero_st
     reference forms from its outputs (tests/test_varlen.py:103), fused into the kernels' epilogues.
     ``save_carry=False`` keeps only q, k, v between the forward and the backward, as the reference does, instead of
     the per-(row, 32-key sub-tile) products (L^2 / 16 bytes per head and sequence); the backward rebuilds them with one
-    more kernel.  Gradients are bit-identical either way."""
+    more kernel.  Gradients are bit-identical either way.
+
+    A ``cu_seqlens`` that exists only on the device (a GPU tensor with ``zero_start=False``, or any call under
+    ``torch.compile``) cannot be validated on the host.  The scheduler kernel validates it instead, and also checks
+    that the sequences fit the scratch sized from ``max_seqlens``; when either check fails it schedules NOTHING:
+    ``o``, ``rem`` and all gradients come back as zeros and no error is raised (the reference reads the same entries
+    unchecked and would run out of bounds, sb_varlen_fwd.py:283-288).  Set ``SBA_DEBUG_CHECK=1`` to have every launch
+    followed by a read of the scheduler's status word (one synchronisation per call) and a ``ValueError`` that says
+    which check failed; never understate ``max_seqlens``."""
     # The lengths are on the host when cu_seqlens was given as a CPU tensor, or after the one device-to-host copy that
     # stands in for the reference's `assert cu_seqlens[0] == 0` (sb_varlen/__init__.py:71-73, the same host sync).
     # They are then validated there and the carry buffer is sized exactly; a device-only cu_seqlens is validated by

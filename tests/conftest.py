@@ -3,6 +3,10 @@ import sys
 
 import pytest
 
+# Every launch made through the Python operators in the tests is followed by a read of the scheduler's status word: a
+# schedule the device refused (or a wait of the chained backward that ran out) raises instead of returning zeros.
+os.environ.setdefault("SBA_DEBUG_CHECK", "1")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PKG_PARENT = os.path.join(ROOT, "stickbreaking-attention_amd")
 for p in (ROOT, PKG_PARENT):

@@ -13,10 +13,11 @@ The adversarial configuration scales q and k by 3.  dq and dk are contractions o
 gradient against k and q (the reference rounds at the same point: sb_varlen_bwd.py:449-450); with |dZ| up to 16
 and |k| ~ 3 that rounding alone puts a handful of elements a few thousandths beyond the bound.  That floor is not
 fitted: the test evaluates `oracle.rounding_floor` (float64 arithmetic, P and dZ rounded to bf16 before their
-contractions, bf16 outputs) on the same inputs and allows the kernels the floor's own largest excess plus 2e-3 for
-the fp32 arithmetic in between.
+contractions, bf16 outputs) on the same inputs and allows the kernels the floor's own largest excess plus
+FLOOR_MARGIN (below) for the fp32 arithmetic in between; every run prints the margin it needed.
 """
 import math
+import os
 
 import numpy as np
 import pytest
@@ -192,6 +193,17 @@ def test_saturated_logits_long_row(gpu_device):
     got = run_varlen(*dev[:3], cu.to(gpu_device), lengths, False, False, dev[3], dev[4])
     for n, a, b in zip(NAMES, got, ref):
         tol_check(n, a, b, torch.bfloat16, "saturated")
+    # row_stat = log2(rem) of a row whose remainder underflows fp32 is -inf (never NaN), where the reference keeps a
+    # finite neg_log_acc; rem is 0 (or a 16-bit denormal) in both.  Wherever the true log2(rem) is within fp32's exponent range it is met.
+    from stickbreaking_attention import _native
+
+    _, rem, stat, _ = _native.forward(*dev[:3], cu.to(gpu_device), False, max(lengths), 128 ** -0.5, False, want_carry=False)
+    stat, true_log2 = stat.double().cpu(), torch.log2(ref[1].double())
+    assert not torch.isnan(stat).any() and (stat <= 0).all()
+    underflowed = torch.isinf(stat)
+    assert underflowed.any() and (rem.float().cpu()[underflowed] < 2.0 ** -126).all() and (true_log2[underflowed] < -126).all()
+    ok = true_log2 > -120
+    torch.testing.assert_close(stat[ok], true_log2[ok], atol=2e-2, rtol=1e-3)
 
 
 def test_known_answers(gpu_device):
@@ -253,16 +265,23 @@ def test_strided_token_major_inputs(gpu_device):
     assert b[0].stride() == thd[0].stride()        # o keeps q's layout (empty_like, sb_varlen_fwd.py:417)
 
 
+# What the kernels may add to the rounding floor's own excess over the bound: the floor rounds P and dZ to bf16 where the
+# kernels do, but sums in float64 where they sum in fp32 and in another order.  The largest margin any configuration has
+# needed is printed by every run; this constant is that record rounded up.
+FLOOR_MARGIN = float(os.environ.get("SBA_TEST_FLOOR_MARGIN", "2e-4"))
+
+
 def _check_against_floor(label, got, floor, exact):
     """The bar of the full-size configurations: max(2e-2, 2^-7 |ref|), plus -- where exact arithmetic with bf16
     matrix operands and bf16 outputs (`oracle.rounding_floor`) itself lands beyond that bound on the same inputs, which
     it does by a few thousandths on a handful of elements of the adversarial configuration -- the floor's largest
-    excess and 2e-3 for the fp32 arithmetic in between (allowed excess = max(floor excess + 2e-3, 0): where the floor
-    is inside the bound by 2e-3 or more, the bound itself applies)."""
+    excess and FLOOR_MARGIN for the fp32 arithmetic in between (allowed excess = max(floor excess + FLOOR_MARGIN, 0):
+    where the floor is inside the bound by that margin or more, the bound itself applies)."""
     for n, a, f, b in zip(NAMES, got, floor, exact):
         floor_excess = ((f - b).abs() - error_bound(b, torch.bfloat16)).max().item()
         print(f"{label} {n}: rounding floor max-abs err {(f - b).abs().max().item():.3e}, largest excess {floor_excess:.3e}", flush=True)
-        tol_check(n, a, b, torch.bfloat16, label, allowed_excess=max(floor_excess + 2e-3, 0.0))
+        worst = tol_check(n, a, b, torch.bfloat16, label, allowed_excess=max(floor_excess + FLOOR_MARGIN, 0.0))
+        print(f"{label} {n}: kernel excess - floor excess = {worst - floor_excess:.3e} (margin allowed {FLOOR_MARGIN:.1e})", flush=True)
 
 
 def _full_size(name, gpu_device, oracle_heads, bwd=True, attend_current=False):
@@ -297,13 +316,12 @@ def test_config2_forward_full_size(gpu_device):
 
 
 def test_config3_full_size(gpu_device):
-    # six of the 32 heads against the oracle, drawn from a seed that changes from day to day and is printed, so
-    # that over time every head gets checked; heads 0 and 31 (first / last XCD) are always among them
-    import datetime
-
-    seed = datetime.date.today().toordinal()
-    heads = sorted({0, 31} | set(int(h) for h in np.random.default_rng(seed).choice(np.arange(1, 31), 4, replace=False)))
-    print(f"c3: oracle heads {heads} (seed {seed})", flush=True)
+    # six of the 32 heads against the oracle: heads 0 and 31 (first / last XCD) and four more, the same on every run.
+    # SBA_TEST_HEAD_SEED draws another four (printed), for coverage of the other heads over time.
+    seed = int(os.environ.get("SBA_TEST_HEAD_SEED", "0"))
+    heads = [0, 8, 9, 21, 22, 31] if seed == 0 else sorted(
+        {0, 31} | set(int(h) for h in np.random.default_rng(seed).choice(np.arange(1, 31), 4, replace=False)))
+    print(f"c3: oracle heads {heads} (SBA_TEST_HEAD_SEED={seed})", flush=True)
     inp, got = _full_size("c3", gpu_device, heads)
     # size-independent property over ALL heads: each sequence on its own (fixed-length entry point) reproduces
     # its slice of the packed result bit for bit

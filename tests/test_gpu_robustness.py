@@ -275,8 +275,8 @@ def test_single_sequence_of_64k_tokens(gpu_device, poisoned):
     """One 65536-token sequence, one head: the length at which the per-(row, 32-key sub-tile) planes the backward works
     from (L^2 / 16 bytes per head each) are the largest buffers in play, sized exactly from the host lengths.  o, rem
     and dq are checked against the row-blocked oracle on the first, a middle and the last 2048 rows (rows are
-    independent in those three); dk and dv, which sum over all rows, against the library's fp32 vector-ALU path on the
-    same values -- a separate implementation pinned by its own oracle tests -- and the forward outputs against it too."""
+    independent in those three), dk and dv against it on the last 2048 keys (which only the last 2048 rows see); dk and
+    dv as a whole, which sum over all rows, against the library's fp32 vector-ALU path on the same values -- a separate implementation pinned by its own oracle tests -- and the forward outputs against it too."""
     from stickbreaking_attention import _native
 
     L, D = 65536, 128
@@ -294,6 +294,10 @@ def test_single_sequence_of_64k_tokens(gpu_device, poisoned):
         ref = orc.stream_rowblocked(q[0], k[0], v[0], do[0], drem[0], rows=(r0, r0 + 2048))
         for n, a, b in zip(NAMES[:3], got[:3], ref[:3]):
             tol_check(n, a[0, r0:r0 + 2048], b[r0:r0 + 2048], torch.bfloat16, f"64k rows {r0}..{r0 + 2047}")
+        if r0 == L - 2048:
+            # the last 2048 keys are seen by the last 2048 rows only, so this row block's dk and dv are complete for them
+            for n, a, b in zip(NAMES[3:], got[3:], ref[3:]):
+                tol_check(n, a[0, r0:], b[r0:], torch.bfloat16, f"64k keys {r0}..{L - 1}")
     f32 = run_varlen(*(t.float() for t in dev[:3]), cu, [L], False, False, dev[3].float(), dev[4].float())
     for n, a, b in zip(NAMES, got, f32):
         tol_check(n, a, b.double().cpu(), torch.bfloat16, "64k vs fp32 path")
