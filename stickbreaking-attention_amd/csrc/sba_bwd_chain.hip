@@ -553,6 +553,8 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
     Tile done_tile = tile;
     int32_t* pub_flag = nullptr;                             // chain flag to publish once this wave's stores have completed
     int pub_count = 0;
+    int claim_v = 0;
+    uint32_t rec_w = 0;
     auto store_results = [&](const Tile& tl) {
       const int tl_len = tl.seq_len, tl_j0 = tl.origin;
       const int64_t tl_tok0 = tl.seq_start;
@@ -656,7 +658,7 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
         }
         CH_T(3)
         // ---- dV += P^T dO of block s-1, or dK += dZ^T Q of block s-2 -------------------------------------------
-        const bool has_w = (out ? has_z : (s >= 1 && s - 1 < n)) && !(kChX & 32);
+        const bool has_w = out ? has_z : (s >= 1 && s - 1 < n);
         const int kw = out ? kz : s - 1;
         if (has_w) {
           const int w_base = (out ? ChLds::kDz : ChLds::kP) + (kw & 1) * ChLds::kStage + tr_off;
@@ -693,23 +695,17 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
           pub_flag = nullptr;
         }
         bool requested = false;
-        // The next tile is claimed late, and all in one slot: the head's cursor, the tile record (a scalar load: the
-        // index is uniform), LDS; everybody reads it three slots later.  The two round trips are exposed, once per tile;
-        // spread over three slots they were not, but every slot of this wave then carried the branches and a full
-        // memory wait where the in-flight values merged.
-        if (c == 3 && s == f.a) {
-          int got = 0;
-          if (lane == 0) got = atomicAdd(p.head_queue + head, 1);
-          const int claim = __builtin_amdgcn_readfirstlane(got);
-          if (claim < n_tiles) {
-            const uint32_t* rec = reinterpret_cast<const uint32_t*>(p.k_tiles + claim);
-            const uint32_t r0 = rec[0], r1 = rec[1], r2 = rec[2], r3 = rec[3], r4 = rec[4], r5 = rec[5];
-            if (lane == 0) {
-              next_lds[0] = (int)r0; next_lds[1] = (int)r1; next_lds[2] = (int)r2;
-              next_lds[3] = (int)r3; next_lds[4] = (int)r4; next_lds[5] = (int)r5;
-            }
+        // The next tile is claimed late and in three slots: the cursor, then the tile record, then LDS.  (Here, where
+        // nothing is in flight, so that the claim's own memory operations cost the other slots no wait.)
+        if (c == 3) {
+          if (s == f.a) { if (lane == 0) claim_v = atomicAdd(p.head_queue + head, 1); }
+          else if (s == f.a + 1) {
+            claim_v = __builtin_amdgcn_readfirstlane(claim_v);
+            if (claim_v < n_tiles && lane < 6) rec_w = reinterpret_cast<const uint32_t*>(p.k_tiles + claim_v)[lane];
+          } else if (s == f.a + 2) {
+            if (lane < 6) next_lds[lane] = (int)rec_w;
+            if (lane == 0) next_lds[8] = claim_v;
           }
-          if (lane == 0) next_lds[8] = claim;
         }
         if (s == f.a + 3) {
           const int ns = __builtin_amdgcn_readfirstlane(next_lds[8]);
