@@ -40,24 +40,6 @@ constexpr int kChQStages = 6, kChDoStages = 5;   // Q rows live from the request
                                                  // (2 slots behind), dO rows to the dV contraction (1 slot behind)
 constexpr int kChMinSlots = 6;                   // slots per tile: the next tile is claimed late (see below)
 constexpr int kChSpinLimit = 1 << 17;
-// Timing experiments only (the results are then wrong): bit 0 = never wait for the tile below, bit 1 = no partial dQ
-// loaded from the chain, bit 2 = no dQ contraction, bit 3 = no row requests (direct-to-LDS loads), bit 4 = no chain stores.
-#ifndef SBA_CH_EXPERIMENT
-#define SBA_CH_EXPERIMENT 0
-#endif
-constexpr int kChX = SBA_CH_EXPERIMENT;
-// Instrumented builds (-DSBA_CH_PROFILE): every wave sums the constant-rate counter over the phases of its slots and
-// adds the sums to a table at the end; sba_debug_chain_profile copies the table out and clears it.
-#ifdef SBA_CH_PROFILE
-__device__ unsigned long long g_chain_prof[8][8];
-#define CH_PROF_DECL unsigned long long prof_[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long prof_t_ = __builtin_amdgcn_s_memtime();
-#define CH_T(i) { const unsigned long long t__ = __builtin_amdgcn_s_memtime(); prof_[i] += t__ - prof_t_; prof_t_ = t__; }
-#define CH_PROF_END(row) if (lane == 0) { for (int i_ = 0; i_ < 8; i_++) atomicAdd(&g_chain_prof[row][i_], prof_[i_]); }
-#else
-#define CH_PROF_DECL
-#define CH_T(i)
-#define CH_PROF_END(row)
-#endif
 
 struct ChLds {   // byte offsets into the dynamic LDS segment
   static constexpr int kRowBytes = lds_stride<128>() * 2;            // 304: padded row of 128 16-bit elements
@@ -326,8 +308,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
     u32x2 cin = {0u, 0u};
 #pragma unroll
     for (int i = 0; i < 16; i++) { beta[i] = 0.f; dzl[i] = 0.f; }
-
-    CH_PROF_DECL
     auto slot_fn = [&](f32x16& s_cur, f32x16& dp_cur, f32x16& s_next, f32x16& dp_next) {
       const bool has_item = s < n, has_b = s >= 1 && s <= n;
       const int q0 = kChRows * (nb - 1 - s);                 // first row of block s (when has_item)
@@ -347,9 +327,7 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
       if (unseen) prod_in = 1.f;
       // The barrier that ends the previous slot is met here, behind this slot's bookkeeping.
       __builtin_amdgcn_sched_barrier(0);
-      CH_T(0)
       if (!first_slot) lds_barrier();
-      CH_T(1)
       first_slot = false;
       if (s == a_slot + 3) {                                 // the next tile, as the claiming wave published it
         const int ns = __builtin_amdgcn_readfirstlane(next_lds[8]);
@@ -393,7 +371,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
           asm volatile("global_store_dwordx2 %0, %1, off" :: "v"(dst), "v"(cv) : "memory");
         }
       }
-      CH_T(2)
       // ---- phase A of block s, with the MFMAs of block s+1 (or of nothing: the last block's go unused) --------
       if (has_item) {
         const float drem = (float)drem_raw;
@@ -443,7 +420,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
           __builtin_amdgcn_sched_barrier(0);
         };
         if (diag) fused(std::true_type{}); else fused(std::false_type{});
-        CH_T(3)
         if (s + 1 < n) advance();                            // (the last block's MFMAs ran on a stage that is not a new block)
         // [row][key] tile: this lane's 16 consecutive keys start at column 32*g + 16*half of row `col`.
         T* p_lds = reinterpret_cast<T*>(lds_raw + ChLds::kP + (s & 1) * ChLds::kStage);
@@ -455,7 +431,7 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
         // replaces it with C below the next tile, and all four waves of the tile read the same slot.
         if (J > 0) {
           bool ok = !row_ok || (cin[1] == (uint32_t)J);
-          if (!(kChX & 1) && !aborted && !__all(ok)) {       // the tile below has not got this far yet
+          if (!aborted && !__all(ok)) {       // the tile below has not got this far yet
             int spins = 0;
             while (true) {
               cin = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(crs, qi * 8, 0, kAuxSc1));
@@ -467,7 +443,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
           }
         }
       }
-      CH_T(4)
       // K/V of the next tile into the same registers, once they have fed their last MFMAs of this tile; the next
       // tile's first scores in the last slot, then the next tile becomes the current one.
       const int kv_slot = n > a_slot + 3 ? n : a_slot + 3;
@@ -485,7 +460,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
       } else {
         ++s;
       }
-      CH_T(5)
     };
     while (true) {
       slot_fn(s_a, dp_a, s_b, dp_b);
@@ -494,7 +468,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
       if (done) break;
     }
     lds_barrier();                                           // the consumers' last slot
-    CH_PROF_END(wave)
   } else {
     // =====================================================================================================
     // Consumer wave c: output `out` (0: dV = P^T dO, 1: dK = dZ^T Q), columns 64*cp .. +63, all 128 keys; and columns
@@ -572,7 +545,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
     };
     bool have_tile = true;
     Tile next_tile = tile;
-    CH_PROF_DECL
     while (have_tile) {
       const Facts f = facts_of(tile);
       const int L = f.L, J = f.J, n = f.n, S = f.S;
@@ -593,7 +565,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
 
       for (int s = 0; s < S; ++s) {
         // ---- top of the slot: everything this wave has in flight completes, then it is published ---------------
-        CH_T(6)
         if (s == 0) {
           // K^T of this tile for the dQ contraction, through the wave's scratch: [32 keys][32 columns] at a time,
           // gathered down the keys by the transpose read.  The previous tile's results leave first (same scratch).
@@ -625,22 +596,21 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
             __builtin_amdgcn_s_waitcnt(0xC07F);              // lgkmcnt(0): the reads are done before the scratch is rewritten
           }
         }
-        CH_T(1)
         // ---- the chain: this wave's 32 columns of the rows of block s-2, as the tile below left them -----------
         const int kz = s - 2;                                // block whose dZ is contracted in this slot
         const bool has_z = kz >= 0 && kz < n;
         const int qz0 = kChRows * (f.nb - 1 - kz);
         const bool final_rows = kz >= n - 4;                 // rows of the tile's own 128-row block: dq leaves
-        const bool chain_in = has_z && J > 0 && !(kChX & 2);
+        const bool chain_in = has_z && J > 0;
         // The partial dQ from the tiles below goes straight into the accumulator of this slot's dQ MFMAs.  The count the
         // tile below has published for this wave's columns was requested at the end of the previous slot; if that was
         // too early the wave polls here.  (Whole-vector bit casts: a bit cast of one element of a vector reads element 0.)
-        const bool do_dq = has_z && !(kChX & 4);
+        const bool do_dq = has_z;
         const bool take_in = do_dq && chain_in;
         u32x4 cin[4];
         int flag_v = 0;
         if (take_in) {
-          if (!(kChX & 1) && !aborted && flag_seen < kz + 1) {
+          if (!aborted && flag_seen < kz + 1) {
             int spins = 0;
             while (true) {
               flag_seen = ch_load_flag(pred_flag);
@@ -656,7 +626,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
           ch_chain_load<64>(cin[2], dqc_voff, dqc_desc, soff); ch_chain_load<96>(cin[3], dqc_voff, dqc_desc, soff);
           ch_flag_request(flag_v, pred_flag);
         }
-        CH_T(3)
         // ---- dV += P^T dO of block s-1, or dK += dZ^T Q of block s-2 -------------------------------------------
         const bool has_w = out ? has_z : (s >= 1 && s - 1 < n);
         const int kw = out ? kz : s - 1;
@@ -684,12 +653,10 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
             for (int nn = 0; nn < 2; nn++)
               acc[m][nn] = Elem<T>::mfma(as_vec8<T>(ch_join(a_lo[1][m], a_hi[1][m])), as_vec8<T>(ch_join(b_lo[1][nn], b_hi[1][nn])), acc[m][nn]);
         }
-        CH_T(4)
         // ---- everything this wave had in flight has landed by now (the rows requested and the partial dQ stored in the
         // previous slot, the partial sums just loaded): the previous slot's rows are published, and only then are the
         // rows three slots ahead requested, so that no wait of this slot is a wait for them ---------------------
         if (take_in) ch_vm_wait<5>(); else ch_vm_wait<0>();     // all but the five loads of the chain just issued
-        CH_T(0)
         if (pub_flag) {
           if (lane == 0) __hip_atomic_store(pub_flag, pub_count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           pub_flag = nullptr;
@@ -720,11 +687,8 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
             slot_idx = ns;                                   // used for the flags of the next tile (read at its start)
           }
         }
-        if (!(kChX & 8)) {
-          if (!rq_next && rq_left == 0 && have_next && s + 3 >= S) { request_from(next_tile); rq_next = true; }
-          if (rq_left > 0 && (s + 3 < n || s + 3 >= S)) { request_rows(); requested = true; }
-        }
-        CH_T(2)
+        if (!rq_next && rq_left == 0 && have_next && s + 3 >= S) { request_from(next_tile); rq_next = true; }
+        if (rq_left > 0 && (s + 3 < n || s + 3 >= S)) { request_rows(); requested = true; }
         // ---- dQ^T (32 columns x 32 rows) += K^T dZ^T over the tile's 128 keys ---------------------------------
         if (do_dq) {
           const int z_base = ChLds::kDz + (kz & 1) * ChLds::kStage + rw_off;
@@ -746,7 +710,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
           if (take_in) {
             if (requested) ch_vm_wait<6>(); else ch_vm_wait<0>();
             ch_chain_landed(cin, flag_v);
-            CH_T(7)
             flag_seen = max(flag_seen, __builtin_amdgcn_readfirstlane(flag_v));
 #pragma unroll
             for (int a4 = 0; a4 < 4; a4++) {
@@ -763,7 +726,7 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
                                 pack2<T>(dq0[4 * a4 + 2] * p.logit_scale, dq0[4 * a4 + 3] * p.logit_scale)};
               __builtin_amdgcn_raw_buffer_store_b64(o2, dq_sink.rsrc, dq_voff + 16 * a4, qz0 * dq_sink.stride_bytes, 0);
             }
-          } else if (!(kChX & 16)) {
+          } else {
 #pragma unroll
             for (int a4 = 0; a4 < 4; a4++) {
               const f32x4 v = {dq0[4 * a4], dq0[4 * a4 + 1], dq0[4 * a4 + 2], dq0[4 * a4 + 3]};
@@ -776,7 +739,6 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
           if (!final_rows) { pub_flag = my_flag; pub_count = kz + 1; }
         }
         if (has_z) bump(cq_stage, kChQStages);
-        CH_T(5)
         lds_barrier();
       }
       pending = true;
@@ -787,17 +749,9 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
     __builtin_amdgcn_s_waitcnt(0x0F70);
     if (pub_flag && lane == 0) __hip_atomic_store(pub_flag, pub_count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     if (pending) store_results(done_tile);
-    CH_PROF_END(4 + wave)
   }
 }
 
-#ifdef SBA_CH_PROFILE
-extern "C" int sba_debug_chain_profile(unsigned long long* out) {
-  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(g_chain_prof), sizeof(unsigned long long) * 64) != hipSuccess) return -1;
-  unsigned long long zero[64] = {0};
-  return hipMemcpyToSymbol(HIP_SYMBOL(g_chain_prof), zero, sizeof(zero)) == hipSuccess ? 0 : -1;
-}
-#endif
 
 template <typename T>
 static hipError_t launch_chain_t(const BwdParams& p_in, int max_tiles, hipStream_t stream) {
