@@ -144,9 +144,11 @@ typedef struct SbaArgs {
                                   (head_dim 128, 16-bit, 16-byte aligned rows, a head count that is a multiple of 8, no
                                   add_remainder) ONE kernel in which the key tiles of a sequence hand the row prefix
                                   sums and the partial dQ to each other through the L2; the two kernels otherwise.
-                                  0: the one kernel where it applies AND is the faster one, which it is while
-                                  max_seqlen * num_heads <= 131072 (measured; in packed mode an overstated max_seqlen
-                                  only costs the faster choice).  Must be the same in sba_workspace_bytes and sba_bwd. */
+                                  0: the one kernel where it applies AND was measured to be the faster one: no
+                                  sequence longer than 256 tokens, or at most 32 heads with (total_tokens / num_seqs) *
+                                  num_heads >= 32768 and max_seqlen * num_heads <= 131072 (in packed mode an overstated
+                                  max_seqlen only costs the faster choice).  Must be the same in sba_workspace_bytes
+                                  and sba_bwd. */
   int32_t reserved0;
 } SbaArgs;
 

@@ -71,11 +71,17 @@ int plan(const SbaArgs* a, Layout* out) {
   L.carry_bytes = align_up((size_t)L.carry_slots_per_head * a->num_heads * sizeof(float), 256);
   size_t chain_bytes = 0;
   L.chain_rows = fixed ? B * T : T;
-  // The one-kernel backward is laid out when it is asked for, or (backward_kernels 0) when it is the faster one: it
-  // wins while the longest sequence gives each of a head's workgroups at most four key tiles of 128 (measured on
-  // 256 compute units: beyond that, the partial dQ a tile finds was written too long ago to still be in the L2).
+  // The one-kernel backward is laid out when it is asked for, or (backward_kernels 0) where it is the faster one.
+  // Measured on 256 compute units with the two backwards alternating in one process (uniform lengths and log-normal
+  // mixes, 8 to 64 heads): it wins by 9-13 % when no sequence exceeds two key tiles (nothing is handed over then), and
+  // by 2-6 % while the sequences give each of a head's workgroups between one and four key tiles of 128 (mean length
+  // x heads >= 32768, longest x heads <= 131072) at up to 32 heads; it loses 2-10 % on sequences of 512-1024 tokens
+  // (two more slots per tile than the dK/dV kernel) and 6-20 % beyond four tiles per workgroup (the partial dQ a
+  // tile finds was written too long ago to still be in the L2).
   const bool chain_shape = a->dtype != SBA_F32 && a->head_dim == 128 && (a->num_heads & 7) == 0 && !a->add_remainder;
-  const bool chain_pays = max_len * a->num_heads <= (int64_t)512 * 256;
+  const int64_t mean_len = fixed ? T : T / B;
+  const bool chain_pays = max_len <= 256 ||
+                          (a->num_heads <= 32 && mean_len * a->num_heads >= 32768 && max_len * a->num_heads <= (int64_t)512 * 256);
   if (chain_shape && (a->backward_kernels == 2 || (a->backward_kernels == 0 && chain_pays))) {
     size_t c = off;
     L.off_chain_zero = c;

@@ -117,16 +117,22 @@ def _bwd_kernels(native, q, lengths, backward_kernels, add_remainder=False, max_
 def test_which_backward_runs(gpu_device, native_checked):
     """The one-kernel backward runs only where it applies; left to the library (0) only where it is the faster one."""
     n = native_checked
-    q = torch.zeros(8, 1024, 128, dtype=torch.bfloat16, device=gpu_device)
-    assert _bwd_kernels(n, q, [1024], 2) == 1
-    assert _bwd_kernels(n, q, [1024], 1) == 2
-    assert _bwd_kernels(n, q, [1024], 0) == 1
-    assert _bwd_kernels(n, q, [1024], 2, add_remainder=True) == 2
-    assert _bwd_kernels(n, q[:7], [1024], 2) == 2                                    # 7 heads
-    assert _bwd_kernels(n, q[..., :64], [1024], 2) == 2                              # head_dim 64 (and unaligned rows)
-    assert _bwd_kernels(n, q.float(), [1024], 2) == 2                                # fp32
+    q = torch.zeros(8, 4096, 128, dtype=torch.bfloat16, device=gpu_device)
+    assert _bwd_kernels(n, q, [4096], 2) == 1
+    assert _bwd_kernels(n, q, [4096], 1) == 2
+    assert _bwd_kernels(n, q, [4096], 0) == 1                                        # mean x heads = 32768, longest x heads <= 131072
+    assert _bwd_kernels(n, q, [1024] * 4, 0) == 2                                    # short sequences: two kernels
+    assert _bwd_kernels(n, q, [1024] * 4, 2) == 1
+    assert _bwd_kernels(n, q, [128] * 32, 0) == 1                                    # nothing to hand over: one kernel
+    assert _bwd_kernels(n, q, [4096], 2, add_remainder=True) == 2
+    assert _bwd_kernels(n, q[:7], [4096], 2) == 2                                    # 7 heads
+    assert _bwd_kernels(n, q[..., :64], [4096], 2) == 2                              # head_dim 64
+    assert _bwd_kernels(n, q.float(), [4096], 2) == 2                                # fp32
     big = torch.zeros(32, 8192, 128, dtype=torch.bfloat16, device=gpu_device)
     assert _bwd_kernels(n, big, [8192], 0) == 2                                      # 8192 * 32 > 131072
     assert _bwd_kernels(n, big, [4096, 4096], 0) == 1
     assert _bwd_kernels(n, big, [4096, 4096], 0, max_seqlen=8192) == 2               # an overstated bound decides
     assert _bwd_kernels(n, big, [8192], 2) == 1
+    wide = torch.zeros(64, 2048, 128, dtype=torch.bfloat16, device=gpu_device)
+    assert _bwd_kernels(n, wide, [2048], 0) == 2                                     # more than 32 heads
+    assert _bwd_kernels(n, wide, [128] * 16, 0) == 1
