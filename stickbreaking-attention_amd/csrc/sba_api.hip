@@ -460,9 +460,18 @@ int sba_bwd(const SbaArgs* a) {
   }
   if (lo < 1) return SBA_ERR_WORKSPACE;
   const int64_t passes = cdiv(a->num_heads, lo), group = cdiv(a->num_heads, passes);
+  // The one-kernel backward's layout is the larger one and is only laid out for head counts it applies to, so a group
+  // size below `lo` need not fit although `lo` does: every pass then takes the two-kernel backward, whose layout grows
+  // with the head count and therefore fits.
+  int32_t kernels = a->backward_kernels;
+  for (int64_t heads : {group, a->num_heads % group}) {
+    c.num_heads = (int32_t)heads;
+    if (heads > 0 && (plan(&c, &L) != SBA_OK || L.bwd_bytes > a->workspace_bytes)) kernels = 1;
+  }
   const size_t es = elem_size(a->dtype);
   for (int64_t h0 = 0; h0 < a->num_heads; h0 += group) {
     c = *a;
+    c.backward_kernels = kernels;
     c.num_heads = (int32_t)(a->num_heads - h0 < group ? a->num_heads - h0 : group);
     for (SbaTensor* t : {&c.q, &c.k, &c.v, &c.d_o, &c.dq, &c.dk, &c.dv})
       if (t->ptr) t->ptr = (char*)t->ptr + h0 * t->stride_head * (int64_t)es;

@@ -103,6 +103,26 @@ def test_chained_backward_fixed_length(gpu_device, native_checked):
             tol_check(name, a[b], r, torch.bfloat16, f"chained fixed-length batch {b}")
 
 
+def test_chained_backward_in_head_groups(gpu_device, native_checked):
+    """A backward workspace too small for all heads: the heads go through in groups, each group a chained launch of its
+    own (its own flags, tags and XCD map); same bits as the single launch."""
+    lengths, H = [1500, 700], 16
+    host, dev_t, cu = small_case(H, 128, lengths, torch.bfloat16, seed=77)
+    whole = grads_varlen(native_checked, 2, dev_t, cu, lengths, False)
+    q = dev_t[0]
+    a = native_checked._base_args(q, cu.to(q.device), False, max(lengths), 1.0, False)
+    for f in ("q", "k", "v", "d_o", "dq", "dk", "dv"):
+        setattr(a, f, native_checked._tensor(q, False))
+    need = native_checked._workspace_bytes(a)[1]
+    try:
+        native_checked.set_backward_workspace_limit(int(need * 0.6))          # two groups of 8 heads
+        grouped = grads_varlen(native_checked, 2, dev_t, cu, lengths, False)
+    finally:
+        native_checked.set_backward_workspace_limit(None)
+    for name, x, y in zip(("dq", "dk", "dv"), grouped, whole):
+        assert torch.equal(x, y), name
+
+
 def _bwd_kernels(native, q, lengths, backward_kernels, add_remainder=False, max_seqlen=None):
     """`sba_bwd_kernels` for a packed call on tensors shaped like `q` (nothing is launched)."""
     cu = torch.tensor(np.cumsum(lengths), dtype=torch.int32, device=q.device)
