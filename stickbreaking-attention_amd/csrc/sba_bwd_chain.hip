@@ -473,6 +473,10 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
     // Consumer wave c: output `out` (0: dV = P^T dO, 1: dK = dZ^T Q), columns 64*cp .. +63, all 128 keys; and columns
     // 32*c .. +31 of dQ^T.
     const int c = wave, out = c >> 1, cp = c & 1;
+    // The consumer waves are the critical path of a slot (the producers wait for them at the slot barrier 30 % of the
+    // time) and share each SIMD with a producer wave: raised issue priority for them is worth 2-3 % of the kernel
+    // (priority 1, 2 or 3, or giving the consumers the lower wave ids instead: all the same, and not additive).
+    __builtin_amdgcn_s_setprio(2);
     f32x16 acc[4][2];
     vec8 kstat[kSteps];                                      // K^T of the tile for columns 32c..: A operand of dQ^T = K^T dZ^T
     int cq_stage = 0, cd_stage = 0;                          // stages of the blocks to contract (Q: 2 behind, dO: 1 behind)
