@@ -147,8 +147,11 @@ typedef struct SbaArgs {
                                   0: the one kernel where it applies AND was measured to be the faster one: no
                                   sequence longer than 256 tokens, or at most 32 heads with (total_tokens / num_seqs) *
                                   num_heads >= 32768 and max_seqlen * num_heads <= 131072 (in packed mode an overstated
-                                  max_seqlen only costs the faster choice).  Must be the same in sba_workspace_bytes
-                                  and sba_bwd. */
+                                  max_seqlen only costs the faster choice).  A head count above 8 that is not a multiple
+                                  of 8 is then split where that pays (long sequences): the largest multiple of 8 through
+                                  the one kernel, the remaining heads through the two, one pass after the other (with
+                                  trace_events, [1] and [2] then bracket the last pass's kernels only).  Must be the
+                                  same in sba_workspace_bytes and sba_bwd. */
   int32_t reserved0;
 } SbaArgs;
 
@@ -232,8 +235,8 @@ int sba_bwd(const SbaArgs* args);
 
 /*
  * How many attention kernels sba_bwd runs for these arguments on the current device when the workspace holds all
- * heads: 1 (the chained kernel, see SbaArgs.backward_kernels) or 2 (dQ, then dK/dV); a negative SBA_ERR_* for
- * arguments sba_bwd would refuse.  Launches nothing.  For callers that attribute the time between trace_events.
+ * heads: 1 (the chained kernel, see SbaArgs.backward_kernels) or 2 (dQ, then dK/dV; also for a call whose heads are
+ * split between the two forms); a negative SBA_ERR_* for arguments sba_bwd would refuse.  Launches nothing.  For callers that attribute the time between trace_events.
  * No counterpart in the reference (it always runs one kernel with atomics and locks, sb_varlen_bwd.py:541-640).
  */
 int sba_bwd_kernels(const SbaArgs* args);

@@ -31,10 +31,13 @@ struct Layout {
   int64_t max_q_tiles, max_k_tiles, carry_slots_per_head;
   size_t off_counts, off_q_tiles, off_k_tiles, off_carry_base, off_prefix, off_drem, off_queue, off_carry;
   size_t fwd_bytes, bwd_bytes, carry_bytes;
+  size_t pass_bytes;                        // what ONE pass over these heads needs (bwd_bytes: what sba_bwd wants, see split_heads)
   // One-kernel backward: its buffers share the prefix plane's region (only one of the two backwards runs).
   int64_t chain_rows;                       // rows per head
   size_t off_chain_zero, chain_zero_bytes;  // {C, tag} per row, the flags and the heads' XCC ids: cleared by every launch
   size_t off_chain_c, off_chain_flags, off_chain_xcc, off_chain_dq;
+  int32_t split_heads;                      // > 0: sba_bwd takes this many heads (a multiple of 8) through the one-kernel
+                                            // backward and the rest through the two kernels
 };
 
 int plan(const SbaArgs* a, Layout* out) {
@@ -98,7 +101,22 @@ int plan(const SbaArgs* a, Layout* out) {
   L.off_queue = off;       off = align_up(off + (size_t)a->num_heads * sizeof(int32_t), 256);      // per-head tile cursors
   // the forward's products, rebuilt inside the backward when the caller did not keep them
   L.off_carry = off;       if (a->recompute_carry) off += L.carry_bytes;
-  L.bwd_bytes = off;
+  L.bwd_bytes = L.pass_bytes = off;
+  // A head count that is not a multiple of 8 (the reference's own benchmarks use 12) cannot run the one-kernel backward,
+  // whose workgroups of a head must share an XCD.  Left to choose, sba_bwd then takes the largest multiple of 8 through
+  // it and the remaining heads through the two kernels, one pass after the other on the stream -- where that pays: two
+  // passes have two tails and two schedules, and on the reference's sweep (12 heads, 4 sequences) the split costs 12 %
+  // at 4096 tokens and 2 % at 8192 and gains 4 % at 12288 and 16384.  The workspace must hold either pass.
+  if (a->backward_kernels == 0 && (a->num_heads & 7) != 0 && a->num_heads > 8 &&
+      mean_len * (a->num_heads & ~7) >= (int64_t)12288 * 8) {
+    SbaArgs c = *a;
+    c.num_heads = a->num_heads & ~7;
+    Layout L8;
+    if (plan(&c, &L8) == SBA_OK && L8.chain_zero_bytes > 0) {
+      L.split_heads = c.num_heads;
+      if (L8.bwd_bytes > L.bwd_bytes) L.bwd_bytes = L8.bwd_bytes;
+    }
+  }
   *out = L;
   return SBA_OK;
 }
@@ -343,7 +361,7 @@ int bwd_pass(const SbaArgs* a, int64_t stat_heads, bool first, bool last) {
   if (a->add_remainder && !a->row_stat) return SBA_ERR_NULL;
   for (const SbaTensor* t : {&a->q, &a->k, &a->v, &a->d_o, &a->dq, &a->dk, &a->dv})
     if (t->ptr && ((uintptr_t)t->ptr % es)) return SBA_ERR_ALIGN;
-  if (!a->workspace || ((uintptr_t)a->workspace & 255) || a->workspace_bytes < L.bwd_bytes) return SBA_ERR_WORKSPACE;
+  if (!a->workspace || ((uintptr_t)a->workspace & 255) || a->workspace_bytes < L.pass_bytes) return SBA_ERR_WORKSPACE;
   hipStream_t stream = (hipStream_t)a->stream;
 
   char* ws = (char*)a->workspace;
@@ -449,14 +467,36 @@ int sba_bwd(const SbaArgs* a) {
   Layout L;
   int st = plan(a, &L);
   if (st != SBA_OK) return st;
-  if (a->workspace_bytes >= L.bwd_bytes || a->num_heads == 1) return bwd_pass(a, a->num_heads, true, true);
+  const size_t es = elem_size(a->dtype);
+  // the heads of a call from h0 on, as a call of their own
+  auto heads_from = [&](int64_t h0, int64_t count) {
+    SbaArgs c = *a;
+    c.num_heads = (int32_t)count;
+    for (SbaTensor* t : {&c.q, &c.k, &c.v, &c.d_o, &c.dq, &c.dk, &c.dv})
+      if (t->ptr) t->ptr = (char*)t->ptr + h0 * t->stride_head * (int64_t)es;
+    if (c.d_rem.ptr) c.d_rem.ptr = (char*)c.d_rem.ptr + h0 * c.d_rem.stride_head * (int64_t)es;
+    if (c.carry) c.carry += h0 * L.carry_slots_per_head;          // slots per head do not depend on the head count
+    if (c.row_stat) c.row_stat += h0 * a->total_tokens;
+    return c;
+  };
+  if (L.split_heads > 0 && a->workspace_bytes >= L.bwd_bytes) {
+    SbaArgs c = heads_from(0, L.split_heads);
+    Layout L8;
+    if (plan(&c, &L8) == SBA_OK && bwd_is_chained(&c, L8)) {      // (the tensors and the device allow the one kernel)
+      if ((st = bwd_pass(&c, a->num_heads, true, false)) != SBA_OK) return st;
+      c = heads_from(L.split_heads, a->num_heads - L.split_heads);
+      c.backward_kernels = 1;
+      return bwd_pass(&c, a->num_heads, false, true);
+    }
+  }
+  if (a->workspace_bytes >= L.pass_bytes || a->num_heads == 1) return bwd_pass(a, a->num_heads, true, true);
   // A workspace smaller than the whole call needs: the heads are independent, so they go through in groups of as many
   // as fit (the per-head planes dominate the workspace), one group after the other on the stream.
   SbaArgs c = *a;
   int64_t lo = 0, hi = a->num_heads;           // largest head count whose layout fits: plan() grows with num_heads
   while (lo < hi) {
     c.num_heads = (int32_t)((lo + hi + 1) / 2);
-    if (plan(&c, &L) == SBA_OK && L.bwd_bytes <= a->workspace_bytes) lo = c.num_heads; else hi = c.num_heads - 1;
+    if (plan(&c, &L) == SBA_OK && L.pass_bytes <= a->workspace_bytes) lo = c.num_heads; else hi = c.num_heads - 1;
   }
   if (lo < 1) return SBA_ERR_WORKSPACE;
   const int64_t passes = cdiv(a->num_heads, lo), group = cdiv(a->num_heads, passes);
@@ -466,18 +506,11 @@ int sba_bwd(const SbaArgs* a) {
   int32_t kernels = a->backward_kernels;
   for (int64_t heads : {group, a->num_heads % group}) {
     c.num_heads = (int32_t)heads;
-    if (heads > 0 && (plan(&c, &L) != SBA_OK || L.bwd_bytes > a->workspace_bytes)) kernels = 1;
+    if (heads > 0 && (plan(&c, &L) != SBA_OK || L.pass_bytes > a->workspace_bytes)) kernels = 1;
   }
-  const size_t es = elem_size(a->dtype);
   for (int64_t h0 = 0; h0 < a->num_heads; h0 += group) {
-    c = *a;
+    c = heads_from(h0, a->num_heads - h0 < group ? a->num_heads - h0 : group);
     c.backward_kernels = kernels;
-    c.num_heads = (int32_t)(a->num_heads - h0 < group ? a->num_heads - h0 : group);
-    for (SbaTensor* t : {&c.q, &c.k, &c.v, &c.d_o, &c.dq, &c.dk, &c.dv})
-      if (t->ptr) t->ptr = (char*)t->ptr + h0 * t->stride_head * (int64_t)es;
-    if (c.d_rem.ptr) c.d_rem.ptr = (char*)c.d_rem.ptr + h0 * c.d_rem.stride_head * (int64_t)es;
-    if (c.carry) c.carry += h0 * L.carry_slots_per_head;          // slots per head do not depend on the head count
-    if (c.row_stat) c.row_stat += h0 * a->total_tokens;
     if ((st = bwd_pass(&c, a->num_heads, h0 == 0, h0 + group >= a->num_heads)) != SBA_OK) return st;
   }
   return SBA_OK;

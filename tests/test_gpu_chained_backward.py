@@ -123,6 +123,21 @@ def test_chained_backward_in_head_groups(gpu_device, native_checked):
         assert torch.equal(x, y), name
 
 
+def test_head_count_not_a_multiple_of_eight_is_split(gpu_device, native_checked):
+    """12 heads (the reference's benchmark shape), left to the library: the first 8 go through the one-kernel backward,
+    the other 4 through the two kernels, one pass after the other -- the same bits as the two parts run on their own."""
+    lengths, H = [12288], 12                 # long enough for the split to pay (and so to be chosen)
+    host, dev_t, cu = small_case(H, 128, lengths, torch.bfloat16, seed=78)
+    auto = grads_varlen(native_checked, 0, dev_t, cu, lengths, False)
+    first = grads_varlen(native_checked, 2, [t[:8] for t in dev_t], cu, lengths, False)
+    rest = grads_varlen(native_checked, 1, [t[8:] for t in dev_t], cu, lengths, False)
+    two = grads_varlen(native_checked, 1, dev_t, cu, lengths, False)
+    for name, a, b, c, d in zip(("dq", "dk", "dv"), auto, first, rest, two):
+        assert torch.equal(a[:8], b), f"{name}: heads 0..7 differ from the chained backward on those heads"
+        assert torch.equal(a[8:], c), f"{name}: heads 8..11 differ from the two-kernel backward on those heads"
+        assert not torch.equal(a[:8], d[:8]) or name == "dv"       # (the split really took the other kernel for them)
+
+
 def _bwd_kernels(native, q, lengths, backward_kernels, add_remainder=False, max_seqlen=None):
     """`sba_bwd_kernels` for a packed call on tensors shaped like `q` (nothing is launched)."""
     cu = torch.tensor(np.cumsum(lengths), dtype=torch.int32, device=q.device)
