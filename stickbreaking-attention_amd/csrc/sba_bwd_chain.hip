@@ -558,6 +558,8 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
       int32_t* const my_flag = p.chain_flags + ((int64_t)head * p.chain_tile_cap + slot_idx) * 8 + c;
       const int32_t* const pred_flag = my_flag - 8;
       int flag_seen = 0;                                     // the tile below's count for this wave's columns, as last read
+      int flag_late = 0;                                     // the same count, requested at the end of a slot for the next one
+      bool late_pending = false;
       // dQ partial sums of this sequence's rows (fp32, [row][128]) and the dq output, addressed per sequence.
       const __amdgpu_buffer_rsrc_t dqc_rs = __builtin_amdgcn_make_buffer_rsrc(
           (void*)(p.chain_dq + ((int64_t)head * p.chain_rows + f.crow) * DH), 0, L * DH * 4, 0x00020000);
@@ -614,6 +616,15 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
         u32x4 cin[4];
         int flag_v = 0;
         if (take_in) {
+          // The count that came with the previous slot's partial sums is a slot old by now, and in half of the slots too
+          // old to cover this block although the tile below has published it since.  A second request, issued just
+          // before the previous slot's four stores (so that waiting for it is not waiting for them), is looked at first:
+          // a poll costs a full round trip, and more than one as a rule.
+          if (!aborted && flag_seen < kz + 1 && late_pending) {
+            ch_vm_wait<4>();
+            asm volatile("" : "+v"(flag_late) :: "memory");
+            flag_seen = max(flag_seen, __builtin_amdgcn_readfirstlane(flag_late));
+          }
           if (!aborted && flag_seen < kz + 1) {
             int spins = 0;
             while (true) {
@@ -630,6 +641,7 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
           ch_chain_load<64>(cin[2], dqc_voff, dqc_desc, soff); ch_chain_load<96>(cin[3], dqc_voff, dqc_desc, soff);
           ch_flag_request(flag_v, pred_flag);
         }
+        late_pending = false;
         // ---- dV += P^T dO of block s-1, or dK += dZ^T Q of block s-2 -------------------------------------------
         const bool has_w = out ? has_z : (s >= 1 && s - 1 < n);
         const int kw = out ? kz : s - 1;
@@ -722,6 +734,7 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
               for (int b = 0; b < 4; b++) dq0[4 * a4 + b] += v[b];
             }
           }
+          if (J > 0 && kz + 1 < n && !aborted) { ch_flag_request(flag_late, pred_flag); late_pending = true; }
           // dq0[4a + b]: row qz0 + col, column 32c + 8a + 4*half + b.
           if (final_rows) {
 #pragma unroll
