@@ -227,8 +227,9 @@ int sba_fwd_static(const SbaArgs* args);
  * "attn_bwd"), and the `locked_add` accumulation (sb_varlen_bwd.py:11-53).
  * Workspace: bwd_bytes of sba_workspace_bytes runs all heads in one pass.  A smaller workspace is taken as a memory
  * limit: the heads are independent, so the call takes them through in groups of as many as fit, one group after
- * the other on the stream (same results).  The minimum is bwd_bytes of the same arguments with num_heads = 1;
- * below that the call returns SBA_ERR_WORKSPACE before launching anything.  With several groups trace_events
+ * the other on the stream (bit-identical results as long as every pass takes the same form of the backward as
+ * the single pass would -- see backward_kernels; equal to rounding otherwise).  The minimum is bwd_bytes of the
+ * same arguments with num_heads = 1; * below that the call returns SBA_ERR_WORKSPACE before launching anything.  With several groups trace_events
  * bracket the whole call but only the last group's dQ / dK/dV split.
  */
 int sba_bwd(const SbaArgs* args);
