@@ -229,7 +229,8 @@ int sba_fwd_static(const SbaArgs* args);
  * limit: the heads are independent, so the call takes them through in groups of as many as fit, one group after
  * the other on the stream (bit-identical results as long as every pass takes the same form of the backward as
  * the single pass would -- see backward_kernels; equal to rounding otherwise).  The minimum is bwd_bytes of the
- * same arguments with num_heads = 1; * below that the call returns SBA_ERR_WORKSPACE before launching anything.  With several groups trace_events
+ * same arguments with num_heads = 1; below that the call returns SBA_ERR_WORKSPACE before launching anything.
+ * With several groups trace_events
  * bracket the whole call but only the last group's dQ / dK/dV split.
  */
 int sba_bwd(const SbaArgs* args);
