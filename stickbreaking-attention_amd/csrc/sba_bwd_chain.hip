@@ -570,7 +570,7 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
       const int dq_voff = col * dq_sink.stride_bytes + (32 * c + 4 * half) * 2;
 
       for (int s = 0; s < S; ++s) {
-        // ---- top of the slot: everything this wave has in flight completes, then it is published ---------------
+        // ---- first slot of a tile: the previous tile's results leave, the tile's K^T is set up --------------------
         if (s == 0) {
           // K^T of this tile for the dQ contraction, through the wave's scratch: [32 keys][32 columns] at a time,
           // gathered down the keys by the transpose read.  The previous tile's results leave first (same scratch).
@@ -608,9 +608,8 @@ __global__ __launch_bounds__(kChThreads) void bwd_chain_kernel(BwdParams p) {
         const int qz0 = kChRows * (f.nb - 1 - kz);
         const bool final_rows = kz >= n - 4;                 // rows of the tile's own 128-row block: dq leaves
         const bool chain_in = has_z && J > 0;
-        // The partial dQ from the tiles below goes straight into the accumulator of this slot's dQ MFMAs.  The count the
-        // tile below has published for this wave's columns was requested at the end of the previous slot; if that was
-        // too early the wave polls here.  (Whole-vector bit casts: a bit cast of one element of a vector reads element 0.)
+        // The partial dQ of the tiles below is requested here and added behind this slot's dQ MFMAs.  The tile below must
+        // have published the block for this wave's columns first: its count is known from earlier readings, or polled.
         const bool do_dq = has_z;
         const bool take_in = do_dq && chain_in;
         u32x4 cin[4];
