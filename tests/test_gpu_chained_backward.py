@@ -81,6 +81,60 @@ def test_chained_backward_matches_oracle_and_two_kernels(gpu_device, native_chec
         assert (diff <= 2 * error_bound(r.double(), dtype)).all(), f"{label}: {name} chained vs two kernels {diff.max().item():.3e}"
 
 
+EDGE_LENGTHS = [1, 2, 31, 32, 33, 63, 64, 65, 96, 97, 127, 128, 129, 160, 161, 191, 192, 193, 255, 256, 257, 300, 385, 511, 513, 640,
+                769, 1025]
+
+
+def draw_chained_case(seed):
+    rng = np.random.default_rng(9000 + seed)
+    n_seq = int(rng.integers(1, 9))
+    return dict(
+        seed=seed, dtype=[torch.bfloat16, torch.bfloat16, torch.float16][rng.integers(0, 3)], H=int(rng.choice([8, 8, 16, 24])),
+        lengths=[int(rng.choice(EDGE_LENGTHS)) if rng.random() < 0.7 else int(rng.integers(1, 1400)) for _ in range(n_seq)],
+        attend_current=bool(rng.integers(0, 2)), zero_start=bool(rng.integers(0, 2)), host_cu=bool(rng.integers(0, 2)),
+        save_carry=bool(rng.integers(0, 3) > 0), token_major=bool(rng.integers(0, 3) == 0), pad=int(rng.choice([0, 0, 1, 130])),
+        qk_std=float(rng.choice([1.0, 1.0, 2.0])), int64_cu=bool(rng.integers(0, 2)),
+    )
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_chained_case_against_oracle(gpu_device, native_checked, seed):
+    """The seeded sweep of test_gpu_random_sweep.py on the shapes the one-kernel backward applies to (head_dim 128, 8 / 16 / 24
+    heads), with that backward forced: ragged lengths around the block and tile edges, attend_current, a leading zero in
+    cu_seqlens, cu_seqlens on the host or the device, rebuilt products, token-major strides, rows no sequence covers."""
+    from stickbreaking_attention import sb_attn_varlen
+
+    c = draw_chained_case(seed)
+    print({k: (str(v) if k == "dtype" else v) for k, v in c.items()}, flush=True)
+    dtype, H, lengths, pad = c["dtype"], c["H"], c["lengths"], c["pad"]
+    T = sum(lengths)
+    g = torch.Generator().manual_seed(9500 + seed)
+    q, k, v, do = (torch.randn(H, T + pad, 128, generator=g) for _ in range(4))
+    drem = torch.randn(H, T + pad, generator=g)
+    q, k = q * c["qk_std"], k * c["qk_std"]
+    host = [t.to(dtype) for t in (q, k, v, do, drem)]
+    ends = torch.tensor(np.cumsum(lengths), dtype=torch.int64 if c["int64_cu"] else torch.int32)
+    cu = torch.cat([torch.zeros(1, dtype=ends.dtype), ends]) if c["zero_start"] else ends
+
+    def to_gpu(t):
+        if c["token_major"] and t.dim() == 3:                      # (T, H, D) storage viewed as (H, T, D)
+            return t.transpose(0, 1).contiguous().to(gpu_device).transpose(0, 1)
+        return t.to(gpu_device)
+
+    native_checked.BACKWARD_KERNELS = 2
+    qd, kd, vd = (to_gpu(t).requires_grad_() for t in host[:3])
+    o, rem = sb_attn_varlen(qd, kd, vd, cu if c["host_cu"] else cu.to(gpu_device), max(lengths), zero_start=c["zero_start"],
+                            attend_current=c["attend_current"], save_carry=c["save_carry"])
+    grads = torch.autograd.grad([o, rem], [qd, kd, vd], [to_gpu(host[3]), host[4].to(gpu_device)])
+    torch.cuda.synchronize()
+    cov = [t[:, :T] for t in host]
+    ref = orc.varlen_stream(*cov[:3], ends, attend_current=c["attend_current"], do=cov[3], drem=cov[4], dtype=torch.float64)
+    for name, a, b in zip(("o", "rem", "dq", "dk", "dv"), (o, rem, *grads), ref):
+        tol_check(name, a[:, :T], b, dtype, f"chained sweep {seed}")
+        if pad:
+            assert (a[:, T:] == 0).all(), f"{name}: rows no sequence covers must be zero"
+
+
 def test_chained_backward_fixed_length(gpu_device, native_checked):
     """`sb_attn` (batch, head, token, head_dim): the chain buffers are addressed per batch element."""
     from stickbreaking_attention import sb_attn
