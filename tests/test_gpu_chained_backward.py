@@ -192,6 +192,33 @@ def test_head_count_not_a_multiple_of_eight_is_split(gpu_device, native_checked)
         assert not torch.equal(a[:8], d[:8]) or name == "dv"       # (the split really took the other kernel for them)
 
 
+def test_benchmark_shape_all_heads_agree_with_two_kernels_and_repeat(gpu_device, native_checked):
+    """The benchmark configuration (32 heads, 32768 tokens, 25 sequences) through both backwards on ALL heads -- every
+    workgroup of every XCD, several tiles per workgroup, where the oracle of test_gpu_parity.py covers six heads: two
+    independent orders of summation must agree to twice the bound each has against the oracle, and the one-kernel
+    backward must repeat its own bits."""
+    import bench
+
+    inp = bench.make_inputs("c3", gpu_device)
+    lengths = inp["lengths"]
+    dev_t = [inp[n] for n in ("q", "k", "v", "do", "drem")]
+    cu = inp["cu"].cpu()
+    assert not inp["zero_start"]
+    two = grads_varlen(native_checked, 1, dev_t, cu, lengths, False)
+    one = grads_varlen(native_checked, 2, dev_t, cu, lengths, False)
+    again = grads_varlen(native_checked, 2, dev_t, cu, lengths, False)
+    for name, a, b, c in zip(("dq", "dk", "dv"), one, two, again):
+        assert torch.isfinite(a.float()).all(), name
+        assert torch.equal(a, c), f"{name} differs between two runs of the chained kernel"
+        worst = -float("inf")
+        for h in range(0, a.shape[0], 8):                     # in slices, to bound the fp32 temporaries
+            x, y = a[h:h + 8].float(), b[h:h + 8].float()
+            excess = (x - y).abs() - 2 * torch.maximum(torch.full_like(y, 2e-2), y.abs() * 2.0 ** -7)
+            worst = max(worst, excess.max().item())
+        print(f"c3 all heads, chained vs two kernels, {name}: largest excess over twice the bound {worst:.3e}", flush=True)
+        assert worst <= 0.0, f"{name}: chained and two-kernel backward differ by {worst:.3e} beyond twice the bound"
+
+
 def _bwd_kernels(native, q, lengths, backward_kernels, add_remainder=False, max_seqlen=None):
     """`sba_bwd_kernels` for a packed call on tensors shaped like `q` (nothing is launched)."""
     cu = torch.tensor(np.cumsum(lengths), dtype=torch.int32, device=q.device)
